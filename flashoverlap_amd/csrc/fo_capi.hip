@@ -1,0 +1,177 @@
+// extern "C" surface of libfo_hip.so (declared in include/flashoverlap_hip.h):
+// argument marshalling only; the kernels and their launchers live in
+// fo_gemm.hip, fo_sync.hip and fo_rmsnorm.hip.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "fo_internal.h"
+
+namespace fo {
+
+static thread_local char t_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_error, sizeof t_error, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// Layout tile selected by each Algo index, in the order of the reference's
+// instance list (src/inc/signal_instances.inc:1-6).  The third number is the
+// reference's k-tile; this library always stages 64 k-elements per LDS stage,
+// so entries that differ only in it select the same kernel.
+static const int kAlgo[][3] = {
+    {128, 128, 32}, {128, 128, 64}, {128, 256, 32}, {128, 256, 64}, {256, 128, 32}, {256, 128, 64},
+};
+constexpr int kAlgoCount = sizeof(kAlgo) / sizeof(kAlgo[0]);
+
+int algo_tile(int algo, int* BM, int* BN, int* BK) {
+    if (algo < 0 || algo >= kAlgoCount) return FO_ERR_ARG;
+    *BM = kAlgo[algo][0];
+    *BN = kAlgo[algo][1];
+    *BK = kAlgo[algo][2];
+    return FO_OK;
+}
+
+}  // namespace fo
+
+using namespace fo;
+
+extern "C" {
+
+int fo_version(void) { return 100; }
+
+const char* fo_last_error(void) { return t_error; }
+
+int fo_algo_count(void) { return kAlgoCount; }
+
+int fo_algo_tile(int algo, int* BM, int* BN, int* BK) {
+    if (!BM || !BN || !BK) return fail(FO_ERR_ARG, "fo_algo_tile: null output");
+    if (algo_tile(algo, BM, BN, BK) != FO_OK) return fail(FO_ERR_ARG, "fo_algo_tile: Algo %d out of range 0..%d", algo, kAlgoCount - 1);
+    return FO_OK;
+}
+
+int fo_device_info(int* cu_count, int* clock_khz, int* xcd_count) {
+    int dev = 0;
+    FO_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    FO_HIP(hipGetDeviceProperties(&prop, dev));
+    if (cu_count) *cu_count = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    if (xcd_count) *xcd_count = 8;  // MI355X: 8 accelerator dies, 32 CUs each
+    return FO_OK;
+}
+
+int fo_gemm(int dtype, int algo, int M, int N, int K, const void* A, const void* B, void* D, void* stream) {
+    return launch_gemm(0, dtype, algo, M, N, K, 1, nullptr, 0, nullptr, A, B, D, nullptr, nullptr, nullptr, 0,
+                       (hipStream_t)stream);
+}
+
+int fo_gemm_signal(int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg_dev, int G,
+                   const int* group_table, const void* A, const void* B, void* D, int* MM, const int* RA,
+                   int monitor, void* stream) {
+    return launch_gemm(1, dtype, algo, M, N, K, rLDN, cseg_dev, G, group_table, A, B, D, MM, RA, nullptr, monitor,
+                       (hipStream_t)stream);
+}
+
+int fo_gemm_scatter(int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg_dev, int G,
+                    const int* group_table, const void* A, const void* B, void* D, int* MM, const int* RA,
+                    const int* RE, int monitor, void* stream) {
+    return launch_gemm(2, dtype, algo, M, N, K, rLDN, cseg_dev, G, group_table, A, B, D, MM, RA, RE, monitor,
+                       (hipStream_t)stream);
+}
+
+int fo_build_group_table(const int* cseg_dev, int G, int T, int* group_table, void* stream) {
+    return launch_group_table(cseg_dev, G, T, group_table, (hipStream_t)stream);
+}
+
+int fo_raster_hint(int algo, int M, int N, int* hint_host) { return raster_hint(algo, M, N, hint_host); }
+
+int fo_wait(int that, int* addr, void* stream) { return launch_wait(that, addr, (hipStream_t)stream); }
+
+int fo_wait_consume(const int* cseg_dev, int G, int* MM, const void* src, void* dst, long long tile_elems,
+                    int nslices, long long slice_stride, int* order_log, int nblocks, void* stream) {
+    return launch_wait_consume(cseg_dev, G, MM, src, dst, tile_elems, nslices, slice_stride, order_log, nblocks,
+                               (hipStream_t)stream);
+}
+
+int fo_set_wait_timeout_ms(int ms) { return set_wait_timeout_ms(ms); }
+
+int fo_wait_timeouts(int* count, int reset) { return wait_timeouts(count, reset); }
+
+int fo_consume(const void* src, void* dst, size_t bytes, void* stream) {
+    return launch_consume(src, dst, bytes, (hipStream_t)stream);
+}
+
+int fo_reorder_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
+                       int rldn, const int* RA, float eps, void* stream) {
+    if (!RA) return fail(FO_ERR_ARG, "fo_reorder_rmsnorm: null RA");
+    return launch_rmsnorm(dtype, x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, (hipStream_t)stream);
+}
+
+int fo_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, float eps, void* stream) {
+    return launch_rmsnorm(dtype, x, gamma, out, bs, dim, 0, 0, 0, nullptr, eps, (hipStream_t)stream);
+}
+
+int fo_stream_create(void** stream) {
+    if (!stream) return fail(FO_ERR_ARG, "fo_stream_create: null output");
+    hipStream_t s;
+    FO_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = (void*)s;
+    return FO_OK;
+}
+
+int fo_stream_destroy(void* stream) {
+    if (stream) FO_HIP(hipStreamDestroy((hipStream_t)stream));
+    return FO_OK;
+}
+
+int fo_stream_sync(void* stream) {
+    FO_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return FO_OK;
+}
+
+int fo_stream_join(void* signaller, void* waiter) {
+    hipEvent_t ev;
+    FO_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    hipError_t e = hipEventRecord(ev, (hipStream_t)signaller);
+    if (e == hipSuccess) e = hipStreamWaitEvent((hipStream_t)waiter, ev, 0);
+    hipError_t d = hipEventDestroy(ev);
+    FO_HIP(e);
+    FO_HIP(d);
+    return FO_OK;
+}
+
+int fo_event_create(void** ev) {
+    if (!ev) return fail(FO_ERR_ARG, "fo_event_create: null output");
+    hipEvent_t e;
+    FO_HIP(hipEventCreate(&e));
+    *ev = (void*)e;
+    return FO_OK;
+}
+
+int fo_event_destroy(void* ev) {
+    if (ev) FO_HIP(hipEventDestroy((hipEvent_t)ev));
+    return FO_OK;
+}
+
+int fo_event_record(void* ev, void* stream) {
+    FO_HIP(hipEventRecord((hipEvent_t)ev, (hipStream_t)stream));
+    return FO_OK;
+}
+
+int fo_event_sync(void* ev) {
+    FO_HIP(hipEventSynchronize((hipEvent_t)ev));
+    return FO_OK;
+}
+
+int fo_event_elapsed_ms(void* start, void* stop, float* ms) {
+    if (!ms) return fail(FO_ERR_ARG, "fo_event_elapsed_ms: null output");
+    FO_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return FO_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,146 @@
+// RMSNorm and reorder+RMSNorm for gfx950: one 64-lane wavefront per output row,
+// the whole row held in registers between the sum of squares and the scaling,
+// 128-bit coalesced HBM accesses, a wavefront butterfly for the reduction (no
+// LDS, no barrier).  The reorder variant gathers the row from the
+// tile-permuted GEMM output: 16 consecutive lanes read one 256-byte row
+// segment of a 128-wide tile, so every access is made of whole cache lines.
+//
+// Arithmetic follows src/rmsnorm/rmsnorm.cuh:62-115 of the reference: fp32 sum
+// of squares, scale = rsqrt(sum/dim + eps), the scaled value rounded to the
+// storage type and then multiplied by gamma in the storage type (the product
+// of two 16-bit floats is exact in fp32, so rounding it once equals the
+// reference's half-precision multiply).  eps is a parameter here.
+#include <hip/hip_runtime.h>
+
+#include "fo_internal.h"
+
+namespace fo {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<_Float16> {
+    using type = f16x8;
+};
+template <>
+struct Vec8<__bf16> {
+    using type = bf16x8;
+};
+
+constexpr int kRowsPerBlock = 4;  // one wavefront per row
+
+// CH = 16-byte chunks per lane (dim <= CH * 512).
+template <typename T, int CH, bool REORDER>
+__global__ void __launch_bounds__(256) rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+                                                      T* __restrict__ out, int bs, int dim, int BM, int BN,
+                                                      int rldn, const int* __restrict__ RA, float eps) {
+    using vec = typename Vec8<T>::type;
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= bs) return;
+
+    const int nchunk = dim >> 3;
+    vec xv[CH];
+    if constexpr (REORDER) {
+        const int ldn = dim / BN;
+        const int tile_row = (row / BM) * ldn;
+        const int in_row = row % BM;
+        const int ld = rldn * BN;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+            const int c = k * 64 + lane;
+            if (c < nchunk) {
+                const int j = c << 3;
+                const int s = RA[tile_row + j / BN];
+                const size_t src = (size_t)((s / rldn) * BM + in_row) * ld + (s % rldn) * BN + j % BN;
+                xv[k] = *(const vec*)(x + src);
+            }
+        }
+    } else {
+        const T* xr = x + (size_t)row * dim;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+            const int c = k * 64 + lane;
+            if (c < nchunk) xv[k] = *(const vec*)(xr + (c << 3));
+        }
+    }
+
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+        if (k * 64 + lane < nchunk) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float f = (float)xv[k][e];
+                ss += f * f;
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    const float scale = rsqrtf(ss / (float)dim + eps);
+
+    T* orow = out + (size_t)row * dim;
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+        const int c = k * 64 + lane;
+        if (c < nchunk) {
+            const vec g = *(const vec*)(gamma + (c << 3));
+            vec o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const T y = (T)((float)xv[k][e] * scale);
+                o[e] = (T)((float)y * (float)g[e]);
+            }
+            *(vec*)(orow + (c << 3)) = o;
+        }
+    }
+}
+
+template <typename T, bool REORDER>
+static int launch_t(const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN, int rldn,
+                    const int* RA, float eps, hipStream_t stream) {
+    const int ch = (dim / 8 + 63) / 64;
+    const dim3 grid((bs + kRowsPerBlock - 1) / kRowsPerBlock), block(64 * kRowsPerBlock);
+#define FO_RMS_CASE(CH)                                                                                   \
+    hipLaunchKernelGGL((rmsnorm_kernel<T, CH, REORDER>), grid, block, 0, stream, (const T*)x, (const T*)gamma, \
+                       (T*)out, bs, dim, BM, BN, rldn, RA, eps)
+    if (ch <= 1) FO_RMS_CASE(1);
+    else if (ch <= 2) FO_RMS_CASE(2);
+    else if (ch <= 4) FO_RMS_CASE(4);
+    else if (ch <= 8) FO_RMS_CASE(8);
+    else if (ch <= 16) FO_RMS_CASE(16);
+    else FO_RMS_CASE(32);
+#undef FO_RMS_CASE
+    FO_HIP(hipGetLastError());
+    return FO_OK;
+}
+
+int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
+                   int rldn, const int* RA, float eps, hipStream_t stream) {
+    const bool reorder = RA != nullptr;
+    const char* who = reorder ? "fo_reorder_rmsnorm" : "fo_rmsnorm";
+    if (dtype != FO_F16 && dtype != FO_BF16) return fail(FO_ERR_ARG, "%s: dtype %d not fp16/bf16", who, dtype);
+    if (bs == 0) return FO_OK;
+    if (!x || !gamma || !out) return fail(FO_ERR_ARG, "%s: null buffer", who);
+    if (bs < 0 || dim <= 0) return fail(FO_ERR_SHAPE, "%s: bs=%d dim=%d", who, bs, dim);
+    if (dim % 8) return fail(FO_ERR_SHAPE, "%s: dim=%d not a multiple of 8", who, dim);
+    if (dim > 32 * 512) return fail(FO_ERR_LIMIT, "%s: dim=%d above the 16384 a wavefront keeps in registers", who, dim);
+    if (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)out) & 15) return fail(FO_ERR_ARG, "%s: buffers must be 16-byte aligned", who);
+    if (reorder) {
+        if (BM <= 0 || BN <= 0 || rldn <= 0) return fail(FO_ERR_ARG, "%s: BM=%d BN=%d rldn=%d", who, BM, BN, rldn);
+        if (BN % 8 || dim % BN) return fail(FO_ERR_SHAPE, "%s: BN=%d must be a multiple of 8 that divides dim=%d", who, BN, dim);
+        if (bs % BM) return fail(FO_ERR_SHAPE, "%s: bs=%d not a multiple of BM=%d", who, bs, BM);
+        if (((long long)(bs / BM) * (dim / BN)) % rldn) return fail(FO_ERR_SHAPE, "%s: rldn=%d must divide the tile count", who, rldn);
+    }
+    if (dtype == FO_F16)
+        return reorder ? launch_t<_Float16, true>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream)
+                       : launch_t<_Float16, false>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream);
+    return reorder ? launch_t<__bf16, true>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream)
+                   : launch_t<__bf16, false>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream);
+}
+
+}  // namespace fo

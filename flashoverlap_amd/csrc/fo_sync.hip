@@ -1,0 +1,201 @@
+// Counter side of the overlap protocol: the wait (counting) kernel, the
+// persistent wait+consume kernel, the consumer copy and the slot->group table.
+//
+// The GEMM epilogue bumps MM[g] with a release-ordered agent-scope atomic once
+// a tile of group g is visible device-wide.  The kernels here run on a second
+// stream while the GEMM is still executing: they poll MM[g] with acquire loads
+// (MI355X has one L2 per XCD and they are not coherent with each other, so the
+// acquire's cache invalidate is what makes the tile data readable), release
+// the group to the consumer once the count is reached, and put the counter
+// back to zero for the next call.  Every wait is bounded in wall-clock time so
+// that a wrong cSeg can delay a stream but never hang the device.
+#include <hip/hip_runtime.h>
+
+#include "fo_internal.h"
+
+namespace fo {
+
+__device__ int g_wait_timeouts = 0;
+
+static int g_timeout_ms = 10000;
+
+// Bounded poll of *addr until pred(value); returns false on expiry.
+template <typename Pred>
+__device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, Pred pred) {
+    const long long t0 = wall_clock64();
+    for (;;) {
+        const int v = __hip_atomic_load(addr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        if (pred(v)) return true;
+        if (wall_clock64() - t0 > ticks) return false;
+        __builtin_amdgcn_s_sleep(8);
+    }
+}
+
+// Counterpart of the reference's kernel_wait_flag (src/wait.cuh:5-9): returns
+// once *addr == that and leaves 0 there.  Nothing else writes *addr between
+// the last tile's signal and the reset, so load-then-store equals the
+// reference's compare-and-swap.
+__global__ void wait_kernel(int that, int* addr, long long ticks) {
+    if (threadIdx.x != 0) return;
+    if (bounded_poll(addr, ticks, [that](int v) { return v == that; }))
+        __hip_atomic_store(addr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        atomicAdd(&g_wait_timeouts, 1);
+}
+
+// Persistent form of the host loop in src/overlap_impl.cu:257-265 (and
+// :312-323 for the ReduceScatter receive layout): walks the groups in index
+// order; all workgroups cooperate on each group's copy.  After its stripe a
+// workgroup bumps MM[g] once more; the workgroup that brings it to
+// cSeg[g] + gridDim.x is the last one out and stores the 0.
+__global__ void __launch_bounds__(256) wait_consume_kernel(const int* __restrict__ cseg, int G, int* MM,
+                                                           const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                           long long tile_units, int nslices,
+                                                           long long slice_stride_units, int* order_log,
+                                                           long long ticks) {
+    __shared__ int s_ok;
+    const int tid = threadIdx.x;
+    long long lo = 0;  // first 16-byte unit of group g in src
+    for (int g = 0; g < G; ++g) {
+        const int need = cseg[g];
+        if (tid == 0) {
+            const bool ok = bounded_poll(MM + g, ticks, [need](int v) { return v >= need; });
+            if (!ok) atomicAdd(&g_wait_timeouts, 1);
+            s_ok = ok;
+        }
+        __syncthreads();
+        if (!s_ok) return;  // uniform: the whole workgroup leaves
+        const long long units = tile_units * need;
+        const long long part = units / nslices;
+        for (int k = 0; k < nslices; ++k) {
+            const uint4* s = src + lo + k * part;
+            uint4* d = dst + k * slice_stride_units + lo / nslices;
+            for (long long i = (long long)blockIdx.x * 256 + tid; i < part; i += (long long)gridDim.x * 256)
+                d[i] = s[i];
+        }
+        __syncthreads();
+        if (tid == 0) {
+            const int old = __hip_atomic_fetch_add(MM + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (old == need + (int)gridDim.x - 1)
+                __hip_atomic_store(MM + g, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (order_log && blockIdx.x == 0) order_log[g] = g;
+        }
+        lo += units;
+    }
+}
+
+__global__ void __launch_bounds__(256) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                      size_t units, const unsigned short* src_tail,
+                                                      unsigned short* dst_tail, int tail) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < units; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+    if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
+}
+
+// table[s] = number of inclusive prefix sums of cseg that are <= s, i.e. what
+// the linear scan in src/overlap/gemm_with_signal.h:188-193 returns.  One
+// workgroup: per-thread run sums, a block scan, then each thread fills the
+// slots of its own run of groups.
+__global__ void __launch_bounds__(1024) group_table_kernel(const int* __restrict__ cseg, int G, int T, int* table) {
+    __shared__ int part[1024];
+    const int tid = threadIdx.x;
+    const int per = (G + 1023) / 1024;
+    const int g0 = tid * per, g1 = min(G, g0 + per);
+    int sum = 0;
+    for (int g = g0; g < g1; ++g) sum += cseg[g];
+    part[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const int add = tid >= off ? part[tid - off] : 0;
+        __syncthreads();
+        part[tid] += add;
+        __syncthreads();
+    }
+    int start = part[tid] - sum;  // exclusive prefix of this thread's run
+    for (int g = g0; g < g1; ++g) {
+        const int n = cseg[g];
+        for (int s = start; s < start + n && s < T; ++s) table[s] = g;
+        start += n;
+    }
+    // Slots beyond sum(cSeg) have no group in the reference (its scan runs off
+    // the array); point them at the last group so a lookup stays in bounds.
+    const int total = part[1023];
+    for (int s = total + tid; s < T; s += 1024) table[s] = G - 1;
+}
+
+static int ticks_for_timeout(long long* ticks) {
+    int dev = 0, khz = 0;
+    FO_HIP(hipGetDevice(&dev));
+    FO_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    if (khz <= 0) khz = 100000;  // the constant 100 MHz counter of gfx9
+    *ticks = (long long)g_timeout_ms * khz;
+    return FO_OK;
+}
+
+int set_wait_timeout_ms(int ms) {
+    if (ms <= 0) return fail(FO_ERR_ARG, "fo_set_wait_timeout_ms: %d ms", ms);
+    g_timeout_ms = ms;
+    return FO_OK;
+}
+
+int wait_timeouts(int* count, int reset) {
+    if (!count) return fail(FO_ERR_ARG, "fo_wait_timeouts: null count");
+    FO_HIP(hipDeviceSynchronize());
+    FO_HIP(hipMemcpyFromSymbol(count, HIP_SYMBOL(g_wait_timeouts), sizeof(int)));
+    if (reset) {
+        const int zero = 0;
+        FO_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_wait_timeouts), &zero, sizeof(int)));
+    }
+    return FO_OK;
+}
+
+int launch_wait(int that, int* addr, hipStream_t stream) {
+    if (!addr) return fail(FO_ERR_ARG, "fo_wait: null counter address");
+    long long ticks;
+    if (int e = ticks_for_timeout(&ticks)) return e;
+    hipLaunchKernelGGL(wait_kernel, dim3(1), dim3(64), 0, stream, that, addr, ticks);
+    FO_HIP(hipGetLastError());
+    return FO_OK;
+}
+
+int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* dst, long long tile_elems,
+                        int nslices, long long slice_stride, int* order_log, int nblocks, hipStream_t stream) {
+    if (!cseg || !MM || !src || !dst) return fail(FO_ERR_ARG, "fo_wait_consume: null argument");
+    if (G <= 0 || nslices <= 0 || tile_elems <= 0) return fail(FO_ERR_ARG, "fo_wait_consume: G=%d nslices=%d tile_elems=%lld", G, nslices, tile_elems);
+    if (nblocks <= 0 || nblocks > 1024) return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d outside 1..1024", nblocks);
+    if (tile_elems % (8LL * nslices)) return fail(FO_ERR_SHAPE, "fo_wait_consume: a tile (%lld elements) must split into %d slices of whole 16-byte units", tile_elems, nslices);
+    if (nslices > 1 && slice_stride % 8) return fail(FO_ERR_SHAPE, "fo_wait_consume: slice_stride=%lld not a multiple of 8 elements", slice_stride);
+    if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_wait_consume: buffers must be 16-byte aligned");
+    long long ticks;
+    if (int e = ticks_for_timeout(&ticks)) return e;
+    hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(256), 0, stream, cseg, G, MM, (const uint4*)src,
+                       (uint4*)dst, tile_elems / 8, nslices, slice_stride / 8, order_log, ticks);
+    FO_HIP(hipGetLastError());
+    return FO_OK;
+}
+
+int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream) {
+    if (bytes == 0) return FO_OK;
+    if (!src || !dst) return fail(FO_ERR_ARG, "fo_consume: null buffer");
+    if (bytes & 1) return fail(FO_ERR_ARG, "fo_consume: %zu bytes is not a whole number of 16-bit elements", bytes);
+    if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_consume: buffers must be 16-byte aligned");
+    const size_t units = bytes / 16;
+    const int tail = (int)((bytes % 16) / 2);
+    size_t blocks = (units + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(consume_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint4*)src, (uint4*)dst,
+                       units, (const unsigned short*)((const char*)src + units * 16),
+                       (unsigned short*)((char*)dst + units * 16), tail);
+    FO_HIP(hipGetLastError());
+    return FO_OK;
+}
+
+int launch_group_table(const int* cseg, int G, int T, int* table, hipStream_t stream) {
+    if (!cseg || !table) return fail(FO_ERR_ARG, "fo_build_group_table: null argument");
+    if (G <= 0 || T <= 0) return fail(FO_ERR_ARG, "fo_build_group_table: G=%d T=%d", G, T);
+    hipLaunchKernelGGL(group_table_kernel, dim3(1), dim3(1024), 0, stream, cseg, G, T, table);
+    FO_HIP(hipGetLastError());
+    return FO_OK;
+}
+
+}  // namespace fo

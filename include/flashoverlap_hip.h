@@ -1,0 +1,179 @@
+/*
+ * flashoverlap_hip.h - C ABI of libfo_hip.so, the gfx950 device library of the
+ * FlashOverlap single-GPU hot path.
+ *
+ * Plain pointers, sizes and opaque stream handles only: no torch types cross
+ * this boundary.  Every entry point returns 0 (FO_OK) or a positive FO_ERR_*
+ * code and never calls exit(); fo_last_error() returns the message of the
+ * last failing call on the calling thread.  All device pointers are on the
+ * current HIP device; `stream` is a hipStream_t passed as void* (NULL = the
+ * null stream).  Nothing here allocates device memory except where stated.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative
+ * to the reference checkout).
+ *
+ * Layout conventions (all row-major, 16-bit elements, K contiguous):
+ *   A [M,K], B [N,K], D = A . B^T.  The "layout tile" is BM x BN as selected
+ *   by `algo` (fo_algo_tile); TM = M/BM, TN = N/BN, T = TM*TN tiles, tile id
+ *   t = m_tile*TN + n_tile, slot s = RA[t].  The permuted output is D viewed
+ *   as [M*N/(rLDN*BN), rLDN*BN] with tile slot s at block-row s/rLDN,
+ *   block-col s%rLDN.
+ */
+#ifndef FLASHOVERLAP_HIP_H
+#define FLASHOVERLAP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum fo_dtype { FO_F16 = 0, FO_BF16 = 1 };
+
+enum fo_status {
+    FO_OK = 0,
+    FO_ERR_ARG = 1,     /* null pointer, bad enum, bad algo index */
+    FO_ERR_SHAPE = 2,   /* shape not supported by the selected tile */
+    FO_ERR_HIP = 3,     /* a HIP runtime call failed */
+    FO_ERR_TIMEOUT = 4, /* a device-side bounded wait gave up */
+    FO_ERR_LIMIT = 5    /* size beyond a documented maximum */
+};
+
+/* ---- library ---------------------------------------------------------- */
+
+int fo_version(void);
+const char* fo_last_error(void);
+
+/* Number of `Algo` indices and the layout tile each one selects.  Replaces the
+ * function-pointer tables indexed by Algo (src/tiling/gemm_tiling.cuh:3-10,
+ * signal_tiling.cuh:3-10, scatter_tiling.cuh:3-10; instances in
+ * src/inc/signal_instances.inc:1-6).  Index order matches the reference:
+ * (128,128,32) (128,128,64) (128,256,32) (128,256,64) (256,128,32) (256,128,64). */
+int fo_algo_count(void);
+int fo_algo_tile(int algo, int* BM, int* BN, int* BK);
+
+/* Device facts used for roofline reports: CU count, clock (kHz), XCD count. */
+int fo_device_info(int* cu_count, int* clock_khz, int* xcd_count);
+
+/* ---- GEMM ------------------------------------------------------------- */
+
+/* D[M,N] = A[M,K] . B[N,K]^T, fp32 accumulate, natural row-major D.
+ * Replaces gemm_func_table[Algo] / mutlass_gemm<TM,TN,TK>
+ * (src/tiling/gemm_dispatcher.h:16-20, src/gemm/gemm.cu:29-113).
+ * Requires M % BM == 0, N % BN == 0, K % 64 == 0, 16-byte aligned pointers. */
+int fo_gemm(int dtype, int algo, int M, int N, int K,
+            const void* A, const void* B, void* D, void* stream);
+
+/* Signalling GEMM.  Tile t is stored at slot RA[t] of the permuted layout and,
+ * after the tile's stores are visible device-wide, MM[group(slot)] is bumped
+ * with a release-ordered atomic.  group(slot) is the index of the first
+ * inclusive prefix sum of cseg_dev[0..G) that exceeds slot.  If `monitor` is
+ * non-zero a ticket is also taken from MM[TN-1] and stored at MM[TN+slot].
+ * Replaces signal_func_table[Algo] / mutlass_gemm_signal<TM,TN,TK>
+ * (src/tiling/gemm_dispatcher.h:7-14, src/overlap/gemm_signal.cu:28-110,
+ * epilogue src/overlap/gemm_with_signal.h:128-202).
+ * group_table: optional device array of T ints, group_table[s] = group(s),
+ * as written by fo_build_group_table; NULL makes every workgroup scan
+ * cseg_dev linearly like the reference (fine for a few dozen groups).
+ * MM must hold at least G ints (TN + T in monitor mode). */
+int fo_gemm_signal(int dtype, int algo, int M, int N, int K, int rLDN,
+                   const int* cseg_dev, int G, const int* group_table,
+                   const void* A, const void* B, void* D,
+                   int* MM, const int* RA, int monitor, void* stream);
+
+/* As fo_gemm_signal, with the row index of the permuted view mapped through
+ * RE (int32, M*N/BN entries) before the store.  Replaces
+ * scatter_func_table[Algo] / mutlass_gemm_scatter<TM,TN,TK>
+ * (src/tiling/gemm_dispatcher.h:22-28, src/overlap/gemm_scatter.cu,
+ * epilogue src/overlap/gemm_with_scatter.h:128-197). */
+int fo_gemm_scatter(int dtype, int algo, int M, int N, int K, int rLDN,
+                    const int* cseg_dev, int G, const int* group_table,
+                    const void* A, const void* B, void* D,
+                    int* MM, const int* RA, const int* RE, int monitor, void* stream);
+
+/* group_table[s] = group(s) for s in [0,T), computed on the device from
+ * cseg_dev.  No counterpart in the reference, whose epilogue rescans cSeg for
+ * every tile (src/overlap/gemm_with_signal.h:188-193); results are identical. */
+int fo_build_group_table(const int* cseg_dev, int G, int T, int* group_table, void* stream);
+
+/* The order in which the GEMM kernels issue layout tiles for this shape:
+ * hint[i] = original tile id of the i-th tile issued (T entries, host memory).
+ * Feeding it to reorder_indices makes slot order equal issue order.  Replaces
+ * the sampled completion order of the reference tuner
+ * (tune/search.py:164-263), which exists because its scheduler is opaque. */
+int fo_raster_hint(int algo, int M, int N, int* hint_host);
+
+/* ---- counting / wait -------------------------------------------------- */
+
+/* Enqueue a one-wave kernel that returns once *addr == that and then stores 0
+ * to *addr.  Replaces launch_kernel_wait_flag (src/wait_launch.h:5,
+ * src/wait_launch.cu:5-7, kernel src/wait.cuh:5-9).  Unlike the reference the
+ * wait is bounded (fo_set_wait_timeout_ms, default 10000 ms): on expiry the
+ * kernel leaves *addr untouched, bumps the timeout count and returns. */
+int fo_wait(int that, int* addr, void* stream);
+
+/* One persistent kernel in place of G (wait, collective) launch pairs: for
+ * g = 0..G-1 in order, wait for MM[g] == cseg_dev[g], copy group g's
+ * contiguous range of `src` (tile_elems * cseg[g] 16-bit elements starting at
+ * tile_elems * sum(cseg[0..g))) to the consumer buffer and reset MM[g].
+ * nslices == 1: dst gets the range at the same offset (the AllReduce
+ * stand-in, src/overlap_impl.cu:257-265).  nslices > 1: the range is cut into
+ * nslices equal parts, part k goes to dst + k*slice_stride + offset/nslices
+ * (the ReduceScatter receive layout, src/overlap_impl.cu:312-323).
+ * order_log (optional, G ints) receives the release sequence.
+ * nblocks workgroups share the groups round-robin (1 = strictly in order). */
+int fo_wait_consume(const int* cseg_dev, int G, int* MM,
+                    const void* src, void* dst, long long tile_elems,
+                    int nslices, long long slice_stride,
+                    int* order_log, int nblocks, void* stream);
+
+int fo_set_wait_timeout_ms(int ms);
+/* Number of bounded waits that expired on the current device since the last
+ * call with reset != 0 (synchronises the device). */
+int fo_wait_timeouts(int* count, int reset);
+
+/* Copy `bytes` bytes (multiple of 2) from src to dst with a device kernel: the
+ * one-GPU stand-in for mcclAllReduce / mcclReduceScatter on one released
+ * group (call sites src/overlap_impl.cu:263, 319-320). */
+int fo_consume(const void* src, void* dst, size_t bytes, void* stream);
+
+/* ---- RMSNorm ---------------------------------------------------------- */
+
+/* out[b,:] = rmsnorm(gather(x)[b,:]) * gamma, gather as in the layout header.
+ * Replaces launch_reorder_rmsnorm_kernel (src/rmsnorm/rmsnorm_launch.h:7-8,
+ * src/rmsnorm/rmsnorm_launch.cu:16-21, kernel src/rmsnorm/rmsnorm.cuh:62-115),
+ * with eps a parameter (the reference fixes 1e-5) and an explicit stream (the
+ * reference uses the null stream).  Requires dim % 8 == 0, BN % 8 == 0. */
+int fo_reorder_rmsnorm(int dtype, const void* x, const void* gamma, void* out,
+                       int bs, int dim, int BM, int BN, int rldn, const int* RA,
+                       float eps, void* stream);
+
+/* Plain row RMSNorm.  Replaces launch_rmsnorm_kernel
+ * (src/rmsnorm/rmsnorm_launch.h:5, src/rmsnorm/rmsnorm.cuh:12-57). */
+int fo_rmsnorm(int dtype, const void* x, const void* gamma, void* out,
+               int bs, int dim, float eps, void* stream);
+
+/* ---- streams and events ----------------------------------------------- */
+
+/* Non-blocking stream at the default priority.  Replaces
+ * musaStreamCreateWithPriority(.., NonBlocking, -5) (src/overlap_impl.cu:146-148). */
+int fo_stream_create(void** stream);
+int fo_stream_destroy(void* stream);
+int fo_stream_sync(void* stream);
+/* Make `waiter` wait for everything enqueued so far on `signaller`.  Replaces
+ * the per-call event create/record/wait/destroy (src/overlap_impl.cu:267-270). */
+int fo_stream_join(void* signaller, void* waiter);
+
+/* Timing helpers for harnesses that cannot use torch events on foreign
+ * streams: opaque hipEvent_t handles. */
+int fo_event_create(void** ev);
+int fo_event_destroy(void* ev);
+int fo_event_record(void* ev, void* stream);
+int fo_event_sync(void* ev);
+int fo_event_elapsed_ms(void* start, void* stop, float* ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHOVERLAP_HIP_H */
