@@ -93,9 +93,10 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host) { return raster_hint(
 int fo_wait(int that, int* addr, void* stream) { return launch_wait(that, addr, (hipStream_t)stream); }
 
 int fo_wait_consume(const int* cseg_dev, int G, int* MM, const void* src, void* dst, long long tile_elems,
-                    int nslices, long long slice_stride, int* order_log, int nblocks, void* stream) {
-    return launch_wait_consume(cseg_dev, G, MM, src, dst, tile_elems, nslices, slice_stride, order_log, nblocks,
-                               (hipStream_t)stream);
+                    int nslices, int slice_first, int slice_count, long long slice_stride, int* order_log,
+                    int nblocks, void* stream) {
+    return launch_wait_consume(cseg_dev, G, MM, src, dst, tile_elems, nslices, slice_first, slice_count,
+                               slice_stride, order_log, nblocks, (hipStream_t)stream);
 }
 
 int fo_set_wait_timeout_ms(int ms) { return set_wait_timeout_ms(ms); }

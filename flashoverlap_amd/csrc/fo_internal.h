@@ -32,7 +32,8 @@ int raster_hint(int algo, int M, int N, int* hint);
 int launch_group_table(const int* cseg, int G, int T, int* table, hipStream_t stream);
 int launch_wait(int that, int* addr, hipStream_t stream);
 int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* dst, long long tile_elems,
-                        int nslices, long long slice_stride, int* order_log, int nblocks, hipStream_t stream);
+                        int nslices, int slice_first, int slice_count, long long slice_stride, int* order_log,
+                        int nblocks, hipStream_t stream);
 int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream);
 int set_wait_timeout_ms(int ms);
 int wait_timeouts(int* count, int reset);

@@ -45,14 +45,17 @@ __global__ void wait_kernel(int that, int* addr, long long ticks) {
 
 // Persistent form of the host loop in src/overlap_impl.cu:257-265 (and
 // :312-323 for the ReduceScatter receive layout): walks the groups in index
-// order; all workgroups cooperate on each group's copy.  After its stripe a
+// order; all workgroups cooperate on each group's copy.  A group's range is
+// cut into nslices equal parts; parts slice_first .. slice_first+slice_count-1
+// are copied, part k to dst + (k - slice_first)*stride + offset/nslices (the
+// receive layout of a ReduceScatter; nslices = 1 is the plain copy).  After its stripe a
 // workgroup bumps MM[g] once more; the workgroup that brings it to
 // cSeg[g] + gridDim.x is the last one out and stores the 0.
 __global__ void __launch_bounds__(256) wait_consume_kernel(const int* __restrict__ cseg, int G, int* MM,
                                                            const uint4* __restrict__ src, uint4* __restrict__ dst,
-                                                           long long tile_units, int nslices,
-                                                           long long slice_stride_units, int* order_log,
-                                                           long long ticks) {
+                                                           long long tile_units, int nslices, int slice_first,
+                                                           int slice_count, long long slice_stride_units,
+                                                           int* order_log, long long ticks) {
     __shared__ int s_ok;
     const int tid = threadIdx.x;
     long long lo = 0;  // first 16-byte unit of group g in src
@@ -67,8 +70,8 @@ __global__ void __launch_bounds__(256) wait_consume_kernel(const int* __restrict
         if (!s_ok) return;  // uniform: the whole workgroup leaves
         const long long units = tile_units * need;
         const long long part = units / nslices;
-        for (int k = 0; k < nslices; ++k) {
-            const uint4* s = src + lo + k * part;
+        for (int k = 0; k < slice_count; ++k) {
+            const uint4* s = src + lo + (slice_first + k) * part;
             uint4* d = dst + k * slice_stride_units + lo / nslices;
             for (long long i = (long long)blockIdx.x * 256 + tid; i < part; i += (long long)gridDim.x * 256)
                 d[i] = s[i];
@@ -158,17 +161,20 @@ int launch_wait(int that, int* addr, hipStream_t stream) {
 }
 
 int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* dst, long long tile_elems,
-                        int nslices, long long slice_stride, int* order_log, int nblocks, hipStream_t stream) {
+                        int nslices, int slice_first, int slice_count, long long slice_stride, int* order_log,
+                        int nblocks, hipStream_t stream) {
     if (!cseg || !MM || !src || !dst) return fail(FO_ERR_ARG, "fo_wait_consume: null argument");
     if (G <= 0 || nslices <= 0 || tile_elems <= 0) return fail(FO_ERR_ARG, "fo_wait_consume: G=%d nslices=%d tile_elems=%lld", G, nslices, tile_elems);
     if (nblocks <= 0 || nblocks > 1024) return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d outside 1..1024", nblocks);
     if (tile_elems % (8LL * nslices)) return fail(FO_ERR_SHAPE, "fo_wait_consume: a tile (%lld elements) must split into %d slices of whole 16-byte units", tile_elems, nslices);
-    if (nslices > 1 && slice_stride % 8) return fail(FO_ERR_SHAPE, "fo_wait_consume: slice_stride=%lld not a multiple of 8 elements", slice_stride);
+    if (slice_first < 0 || slice_count <= 0 || slice_first + slice_count > nslices)
+        return fail(FO_ERR_ARG, "fo_wait_consume: slices [%d, %d) outside 0..%d", slice_first, slice_first + slice_count, nslices);
+    if (slice_count > 1 && slice_stride % 8) return fail(FO_ERR_SHAPE, "fo_wait_consume: slice_stride=%lld not a multiple of 8 elements", slice_stride);
     if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_wait_consume: buffers must be 16-byte aligned");
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
     hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(256), 0, stream, cseg, G, MM, (const uint4*)src,
-                       (uint4*)dst, tile_elems / 8, nslices, slice_stride / 8, order_log, ticks);
+                       (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }

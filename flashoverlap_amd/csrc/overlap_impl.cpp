@@ -1,0 +1,238 @@
+// Host orchestration of the overlapped path on one MI355X.  Follows the call
+// structure of the reference's src/overlap_impl.cu (GEMM on the caller's
+// stream, a per-group wait -> collective loop on a second stream, an event
+// join back), with the collective replaced by a consumer copy into a staging
+// buffer and every failure reported through TORCH_CHECK instead of exit().
+#include "overlap_impl.h"
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include "host_common.h"
+
+OverlapImpl::OverlapImpl() = default;
+
+OverlapImpl::~OverlapImpl() {
+    if (comm_stream_) fo_stream_destroy(comm_stream_);
+}
+
+void OverlapImpl::MutlassInit() {
+    // Like the reference, the stream that is current now is used for every
+    // later GEMM of this object (src/overlap_impl.cu:38-40).
+    gemm_stream_ = (void*)c10::hip::getCurrentHIPStream().stream();
+    gemm_ready_ = true;
+}
+
+void OverlapImpl::McclInit(int64_t tp_rank, int64_t tp_size, std::vector<int64_t> tp_id) {
+    TORCH_CHECK(tp_size >= 1 && tp_rank >= 0 && tp_rank < tp_size, "mccl_init: rank ", tp_rank, " of ", tp_size);
+    TORCH_CHECK(tp_id.size() == 16, "mccl_init: the id must have 16 entries, got ", tp_id.size());
+    // One GPU: no communicator is created (the reference also skips it for
+    // size 1, src/overlap_impl.cu:65-68).  A size above 1 only selects the
+    // ReduceScatter slicing that a rank of that world would see.
+    my_rank_ = tp_rank;
+    my_size_ = tp_size;
+}
+
+void OverlapImpl::OverlapInit() {
+    if (!comm_stream_) FO_CALL(fo_stream_create(&comm_stream_));
+}
+
+void OverlapImpl::SetConsumerMode(int64_t mode) {
+    TORCH_CHECK(mode >= 0 && mode <= 2, "set_consumer_mode: 0 (auto), 1 (per group) or 2 (persistent), got ", mode);
+    consumer_mode_ = mode;
+}
+
+void OverlapImpl::SetConsumerBlocks(int64_t blocks) {
+    TORCH_CHECK(blocks >= 1 && blocks <= 1024, "set_consumer_blocks: 1..1024, got ", blocks);
+    consumer_blocks_ = blocks;
+}
+
+at::Tensor OverlapImpl::Staging() const {
+    TORCH_CHECK(staging_.defined(), "staging: no all-reduce style call has run yet");
+    return staging_;
+}
+
+void OverlapImpl::require_gemm() const {
+    TORCH_CHECK(gemm_ready_, "OverlapImpl: call mutlass_init() first");
+}
+
+void OverlapImpl::require_overlap() const {
+    require_gemm();
+    TORCH_CHECK(comm_stream_ != nullptr, "OverlapImpl: call overlap_init() first");
+}
+
+at::Tensor& OverlapImpl::staging_like(const at::Tensor& C) {
+    if (!staging_.defined() || staging_.numel() != C.numel() || staging_.scalar_type() != C.scalar_type() ||
+        staging_.device() != C.device())
+        staging_ = at::empty({C.numel()}, C.options());
+    return staging_;
+}
+
+const int* OverlapImpl::group_table_for(const at::Tensor& cseg_cpu, const at::Tensor& cseg_gpu, int T) {
+    const int G = (int)cseg_cpu.numel();
+    const int* host = cseg_cpu.data_ptr<int>();
+    std::vector<int> key(host, host + G);
+    key.push_back(T);
+    const bool same_device = group_table_.defined() && group_table_.device() == cseg_gpu.device();
+    if (!same_device || key != table_key_) {
+        group_table_ = at::empty({T}, cseg_gpu.options());
+        FO_CALL(fo_build_group_table(cseg_gpu.data_ptr<int>(), G, T, group_table_.data_ptr<int>(), gemm_stream_));
+        table_key_ = std::move(key);
+    }
+    return group_table_.data_ptr<int>();
+}
+
+void OverlapImpl::bulk_consume(const void* src, void* dst, size_t bytes) {
+    FO_CALL(fo_consume(src, dst, bytes, gemm_stream_));
+}
+
+void OverlapImpl::Gemm(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo) {
+    require_gemm();
+    const fo_host::GemmShape s = fo_host::check_gemm(A, B, C, "mutlass_gemm");
+    c10::DeviceGuard guard(A.device());
+    FO_CALL(fo_gemm(s.dtype, (int)Algo, s.M, s.N, s.K, A.data_ptr(), B.data_ptr(), C.data_ptr(), gemm_stream_));
+}
+
+// Per-group release: either the reference's host loop (one wait kernel and one
+// consumer launch per group, src/overlap_impl.cu:257-265 / 312-323) or one
+// persistent kernel that does the same walk on the device.
+void OverlapImpl::consume_groups(const at::Tensor& C, void* dst, int64_t tile_elems, const at::Tensor& cseg_cpu,
+                                 const at::Tensor& cseg_gpu, at::Tensor& MM, int nslices, int64_t slice_stride) {
+    const int G = (int)cseg_cpu.numel();
+    const int* cseg = cseg_cpu.data_ptr<int>();
+    const int slice_first = slice_stride ? 0 : (int)my_rank_;      // stride 0: only this rank's slice
+    const int slice_count = slice_stride ? nslices : 1;
+    const bool persistent = consumer_mode_ == 2 || (consumer_mode_ == 0 && G > 32);
+    if (persistent) {
+        FO_CALL(fo_wait_consume(cseg_gpu.data_ptr<int>(), G, MM.data_ptr<int>(), C.data_ptr(), dst, tile_elems,
+                                nslices, slice_first, slice_count, slice_stride, nullptr, (int)consumer_blocks_,
+                                comm_stream_));
+        return;
+    }
+    const size_t esz = C.element_size();
+    const char* src = (const char*)C.data_ptr();
+    int64_t acc = 0;
+    for (int g = 0; g < G; ++g) {
+        const int64_t comm = tile_elems * cseg[g];
+        FO_CALL(fo_wait(cseg[g], MM.data_ptr<int>() + g, comm_stream_));
+        const int64_t part = comm / nslices;
+        for (int k = 0; k < slice_count; ++k)
+            FO_CALL(fo_consume(src + (acc + (slice_first + k) * part) * esz,
+                               (char*)dst + (k * slice_stride + acc / nslices) * esz, part * esz, comm_stream_));
+        acc += comm;
+    }
+}
+
+void OverlapImpl::GemmAllReduceOverlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor MM, at::Tensor RA,
+                                       int64_t rLDN, at::Tensor cSEG_CPU, at::Tensor cSEG_GPU, int64_t Algo,
+                                       bool if_monitor) {
+    require_overlap();
+    const fo_host::GemmShape s = fo_host::check_gemm(A, B, C, "gemm_allreduce_overlap");
+    const fo_host::SignalShape g =
+        fo_host::check_signal(s, MM, RA, at::Tensor(), rLDN, cSEG_CPU, cSEG_GPU, (int)Algo, if_monitor, 1,
+                              "gemm_allreduce_overlap");
+    c10::DeviceGuard guard(A.device());
+    at::Tensor& staging = staging_like(C);
+    const int* table = group_table_for(cSEG_CPU, cSEG_GPU, g.T);
+    FO_CALL(fo_gemm_signal(s.dtype, (int)Algo, s.M, s.N, s.K, (int)rLDN, cSEG_GPU.data_ptr<int>(), g.G, table,
+                           A.data_ptr(), B.data_ptr(), C.data_ptr(), MM.data_ptr<int>(), RA.data_ptr<int>(),
+                           if_monitor ? 1 : 0, gemm_stream_));
+    consume_groups(C, staging.data_ptr(), (int64_t)g.BM * g.BN, cSEG_CPU, cSEG_GPU, MM, 1, 0);
+    // The caller's stream continues only after the last group is consumed
+    // (src/overlap_impl.cu:267-270).
+    FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
+}
+
+void OverlapImpl::GemmReduceScatterOverlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D, at::Tensor MM,
+                                           at::Tensor RA, at::Tensor RE, int64_t rLDN, at::Tensor cSEG_CPU,
+                                           at::Tensor cSEG_GPU, int64_t Algo, bool if_monitor) {
+    require_overlap();
+    const fo_host::GemmShape s = fo_host::check_gemm(A, B, C, "gemm_reducescatter_overlap");
+    const fo_host::SignalShape g =
+        fo_host::check_signal(s, MM, RA, RE, rLDN, cSEG_CPU, cSEG_GPU, (int)Algo, if_monitor, (int)my_size_,
+                              "gemm_reducescatter_overlap");
+    const int64_t total = (int64_t)s.M * s.N;
+    fo_host::check_buffer(D, C, "gemm_reducescatter_overlap", "D");
+    // D is one rank's receive buffer [M/ws, N] as in the reference, or all ws
+    // of them stacked [ws, M/ws, N].
+    TORCH_CHECK(D.numel() == total / my_size_ || D.numel() == total,
+                "gemm_reducescatter_overlap: D must hold M*N/world_size = ", total / my_size_, " or M*N = ", total,
+                " elements, got ", D.numel());
+    c10::DeviceGuard guard(A.device());
+    const int* table = group_table_for(cSEG_CPU, cSEG_GPU, g.T);
+    FO_CALL(fo_gemm_scatter(s.dtype, (int)Algo, s.M, s.N, s.K, (int)rLDN, cSEG_GPU.data_ptr<int>(), g.G, table,
+                            A.data_ptr(), B.data_ptr(), C.data_ptr(), MM.data_ptr<int>(), RA.data_ptr<int>(),
+                            RE.data_ptr<int>(), if_monitor ? 1 : 0, gemm_stream_));
+    const int64_t stride = (D.numel() == total && my_size_ > 1) ? total / my_size_ : 0;
+    consume_groups(C, D.data_ptr(), (int64_t)g.BM * g.BN, cSEG_CPU, cSEG_GPU, MM, (int)my_size_, stride);
+    FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
+}
+
+void OverlapImpl::GemmAllReduce(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo) {
+    Gemm(A, B, C, Algo);
+    McclAllReduce(C);
+}
+
+void OverlapImpl::GemmReduceScatter(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D, int64_t Algo) {
+    Gemm(A, B, C, Algo);
+    fo_host::check_buffer(D, C, "gemm_reducescatter", "D");
+    const int64_t recv = C.numel() / my_size_;
+    TORCH_CHECK(D.numel() >= recv, "gemm_reducescatter: D holds ", D.numel(), " elements, needs ", recv);
+    c10::DeviceGuard guard(C.device());
+    // What this rank would receive (src/overlap_impl.cu:104-107), without the sum over ranks.
+    bulk_consume((const char*)C.data_ptr() + my_rank_ * recv * C.element_size(), D.data_ptr(),
+                 recv * C.element_size());
+}
+
+void OverlapImpl::GemmAll2All(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D, int64_t Algo,
+                              at::Tensor mLen_CPU) {
+    TORCH_CHECK(my_size_ == 1, "gemm_all2all: exchanging rows with ", my_size_ - 1,
+                " peers needs more than one GPU, which this build does not drive");
+    Gemm(A, B, C, Algo);  // a world of one sends and receives nothing (src/overlap_impl.cu:132-143)
+}
+
+void OverlapImpl::McclAllReduce(at::Tensor C) {
+    require_gemm();
+    fo_host::check_buffer(C, C, "mccl_allreduce", "C");
+    c10::DeviceGuard guard(C.device());
+    at::Tensor& staging = staging_like(C);
+    bulk_consume(C.data_ptr(), staging.data_ptr(), C.numel() * C.element_size());
+}
+
+void OverlapImpl::SegAllReduce(at::Tensor C, at::Tensor cSEG_CPU, int64_t SegNum) {
+    require_gemm();
+    fo_host::check_buffer(C, C, "seg_allreduce", "C");
+    TORCH_CHECK(cSEG_CPU.device().is_cpu() && cSEG_CPU.scalar_type() == at::kInt && cSEG_CPU.is_contiguous(),
+                "seg_allreduce: cSEG_CPU must be a contiguous int32 host tensor");
+    TORCH_CHECK(SegNum > 0 && C.numel() % SegNum == 0, "seg_allreduce: SegNum=", SegNum, " must divide M*N");
+    c10::DeviceGuard guard(C.device());
+    at::Tensor& staging = staging_like(C);
+    const int* cseg = cSEG_CPU.data_ptr<int>();
+    const int64_t unit = C.numel() / SegNum;
+    int64_t acc = 0;
+    // src/overlap_impl.cu:160-173: cSEG_CPU[s] counts units of M*N/SegNum.
+    for (int64_t sidx = 0; sidx < cSEG_CPU.numel() && acc < C.numel(); ++sidx) {
+        const int64_t n = unit * cseg[sidx];
+        TORCH_CHECK(n >= 0 && acc + n <= C.numel(), "seg_allreduce: segments exceed M*N");
+        bulk_consume((const char*)C.data_ptr() + acc * C.element_size(),
+                     (char*)staging.data_ptr() + acc * C.element_size(), n * C.element_size());
+        acc += n;
+    }
+}
+
+void OverlapImpl::McclReduceScatter(at::Tensor C) {
+    require_gemm();
+    fo_host::check_buffer(C, C, "mccl_reducescatter", "C");
+    c10::DeviceGuard guard(C.device());
+    // In place in the reference: the rank's part of C receives the sum
+    // (src/overlap_impl.cu:183-186).  Stand-in: that part goes to staging.
+    at::Tensor& staging = staging_like(C);
+    const int64_t recv = C.numel() / my_size_;
+    const size_t off = my_rank_ * recv * C.element_size();
+    bulk_consume((const char*)C.data_ptr() + off, (char*)staging.data_ptr() + off, recv * C.element_size());
+}
+
+void OverlapImpl::McclAll2All(at::Tensor C, at::Tensor D, at::Tensor mLen_CPU) {
+    TORCH_CHECK(my_size_ == 1, "mccl_all2all: exchanging rows with ", my_size_ - 1,
+                " peers needs more than one GPU, which this build does not drive");
+}

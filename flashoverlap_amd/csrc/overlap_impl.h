@@ -1,0 +1,79 @@
+// OverlapImpl: host orchestration of the overlapped GEMM + per-group consumer,
+// with the method set of the reference class (src/overlap_impl.h:9-40) so that
+// torch.classes.flashoverlap_class.OverlapImpl is a drop-in on one MI355X.
+//
+// The device is reached only through the C ABI in flashoverlap_hip.h; torch is
+// used for tensor plumbing (pointers, dtype, the caller's current stream) and
+// for the two device buffers this object owns (the staging buffer that stands
+// in for the collective's destination, and the slot->group table).
+#pragma once
+
+#include <ATen/ATen.h>
+#include <torch/custom_class.h>
+
+#include <cstdint>
+#include <vector>
+
+class OverlapImpl : public torch::CustomClassHolder {
+  public:
+    OverlapImpl();
+    ~OverlapImpl() override;
+
+    // src/overlap_impl.cu:38-40, 57-70, 146-148
+    void MutlassInit();
+    void McclInit(int64_t tp_rank, int64_t tp_size, std::vector<int64_t> tp_id);
+    void OverlapInit();
+
+    // src/overlap_impl.cu:42-55
+    void Gemm(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo);
+
+    // src/overlap_impl.cu:221-271, 273-328
+    void GemmAllReduceOverlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor MM, at::Tensor RA, int64_t rLDN,
+                              at::Tensor cSEG_CPU, at::Tensor cSEG_GPU, int64_t Algo, bool if_monitor);
+    void GemmReduceScatterOverlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D, at::Tensor MM,
+                                  at::Tensor RA, at::Tensor RE, int64_t rLDN, at::Tensor cSEG_CPU,
+                                  at::Tensor cSEG_GPU, int64_t Algo, bool if_monitor);
+
+    // src/overlap_impl.cu:72-144 (GEMM followed by one bulk collective, no overlap)
+    void GemmAllReduce(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo);
+    void GemmReduceScatter(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D, int64_t Algo);
+    void GemmAll2All(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D, int64_t Algo, at::Tensor mLen_CPU);
+
+    // src/overlap_impl.cu:150-219
+    void SegAllReduce(at::Tensor C, at::Tensor cSEG_CPU, int64_t SegNum);
+    void McclAllReduce(at::Tensor C);
+    void McclReduceScatter(at::Tensor C);
+    void McclAll2All(at::Tensor C, at::Tensor D, at::Tensor mLen_CPU);
+
+    // ---- additions (no counterpart in the reference) ----
+    // Destination of the AllReduce stand-in: a flat buffer of the size of the
+    // last C passed to an all-reduce style call.
+    at::Tensor Staging() const;
+    // 0 = automatic (per-group launches up to 32 groups, one persistent kernel
+    // beyond), 1 = one (wait, consume) launch pair per group like the
+    // reference's host loop, 2 = one persistent wait+consume kernel.
+    void SetConsumerMode(int64_t mode);
+    // Workgroups of the persistent consumer (default 8).
+    void SetConsumerBlocks(int64_t blocks);
+
+  private:
+    void* gemm_stream_ = nullptr;
+    void* comm_stream_ = nullptr;
+    bool gemm_ready_ = false;
+    int64_t my_rank_ = 0;
+    int64_t my_size_ = 1;
+    int64_t consumer_mode_ = 0;
+    int64_t consumer_blocks_ = 8;
+
+    at::Tensor staging_;
+    at::Tensor group_table_;
+    std::vector<int> table_key_;  // cSeg contents + T the table was built for
+
+    void require_gemm() const;
+    void require_overlap() const;
+    at::Tensor& staging_like(const at::Tensor& C);
+    const int* group_table_for(const at::Tensor& cseg_cpu, const at::Tensor& cseg_gpu, int T);
+    void consume_groups(const at::Tensor& C, void* dst, int64_t tile_elems, const at::Tensor& cseg_cpu,
+                        const at::Tensor& cseg_gpu, at::Tensor& MM, int nslices, int64_t slice_stride);
+    void bulk_consume(const void* src, void* dst, size_t bytes);
+};

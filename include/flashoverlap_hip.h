@@ -116,16 +116,20 @@ int fo_wait(int that, int* addr, void* stream);
 /* One persistent kernel in place of G (wait, collective) launch pairs: for
  * g = 0..G-1 in order, wait for MM[g] == cseg_dev[g], copy group g's
  * contiguous range of `src` (tile_elems * cseg[g] 16-bit elements starting at
- * tile_elems * sum(cseg[0..g))) to the consumer buffer and reset MM[g].
- * nslices == 1: dst gets the range at the same offset (the AllReduce
- * stand-in, src/overlap_impl.cu:257-265).  nslices > 1: the range is cut into
- * nslices equal parts, part k goes to dst + k*slice_stride + offset/nslices
- * (the ReduceScatter receive layout, src/overlap_impl.cu:312-323).
- * order_log (optional, G ints) receives the release sequence.
- * nblocks workgroups share the groups round-robin (1 = strictly in order). */
+ * tile_elems * sum(cseg[0..g))) to the consumer buffer, then reset MM[g].
+ * The range is cut into nslices equal parts; parts slice_first ..
+ * slice_first+slice_count-1 are copied, part k to
+ * dst + (k - slice_first)*slice_stride + offset/nslices.  nslices == 1 copies
+ * the range to the same offset of dst (the AllReduce stand-in,
+ * src/overlap_impl.cu:257-265); nslices == world size with one slice is what a
+ * rank receives from the per-group ReduceScatter (src/overlap_impl.cu:312-323),
+ * with all slices it is every rank's receive buffer side by side.
+ * order_log (optional, G ints) receives the release sequence.  All nblocks
+ * workgroups cooperate on every group, so groups are released strictly in
+ * index order. */
 int fo_wait_consume(const int* cseg_dev, int G, int* MM,
                     const void* src, void* dst, long long tile_elems,
-                    int nslices, long long slice_stride,
+                    int nslices, int slice_first, int slice_count, long long slice_stride,
                     int* order_log, int nblocks, void* stream);
 
 int fo_set_wait_timeout_ms(int ms);

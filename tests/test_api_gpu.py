@@ -1,0 +1,188 @@
+"""GPU tests of the torch-visible API, written the way the reference's own
+scripts drive it (test/test.py:126-197, example/correctness_ar.py:99-127,
+example/correctness_rs.py:100-142, example/RMSNorm.py:23-37), on one GPU."""
+import numpy as np
+import pytest
+import torch
+
+import flashoverlap_amd
+from flashoverlap_amd import capi, tiling
+from oracle import fo_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def api(dev):
+    flashoverlap_amd.load()
+    capi.check(capi.lib().fo_set_wait_timeout_ms(5000))
+    return torch.classes.flashoverlap_class
+
+
+def _overlap(api, rank=0, size=1):
+    o = api.OverlapImpl()
+    o.mccl_init(rank, size, torch.ops.flashoverlap_op.generate_mccl_id())
+    o.mutlass_init()
+    o.overlap_init()
+    return o
+
+
+def _timeouts():
+    import ctypes
+    n = ctypes.c_int()
+    capi.check(capi.lib().fo_wait_timeouts(ctypes.byref(n), 1))
+    return n.value
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_mutlass_and_mublas_gemm(api, dev, dt):
+    M, N, K = 512, 768, 256
+    g = torch.Generator().manual_seed(0)
+    A = torch.randint(-2, 3, (M, K), generator=g).to(dt).to(dev)
+    B = torch.randint(-2, 3, (N, K), generator=g).to(dt).to(dev)
+    want = O.gemm(A.cpu(), B.cpu())
+    o = _overlap(api)
+    C = torch.empty(M, N, dtype=dt, device=dev)
+    o.mutlass_gemm(A, B, C, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(C.cpu(), want)
+    b = api.BaselineImpl()
+    b.mccl_init(0, 1, torch.ops.flashoverlap_op.generate_mccl_id())
+    b.mublas_init()
+    C2 = torch.empty(M, N, dtype=dt, device=dev)
+    b.mublas_gemm(A, B, C2)
+    b.gemm_allreduce(A, B, C2)
+    torch.cuda.synchronize()
+    assert torch.equal(C2.cpu(), want)
+    assert torch.equal(b.staging().cpu().view(M, N), want)
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+def test_allreduce_overlap_like_correctness_ar(api, dev, mode):
+    """All-ones A and B as in example/correctness_ar.py:104-106: every C element
+    is K, so only the permutation and the norm are exercised; then seeded
+    random inputs so the GEMM is exercised too."""
+    M, N, K, algo = 1024, 1024, 1024, 1
+    BM, BN, _ = capi.algo_tile(algo)
+    TM, TN = M // BM, N // BN
+    T = TM * TN
+    hint = tiling.raster_hint(M, N, algo)
+    cseg = tiling.uniform_cseg(T, 4)                       # 16 groups, more than TN = 8
+    cSeg_CPU = torch.tensor(cseg, dtype=torch.int32)
+    cSeg_GPU = cSeg_CPU.to(dev)
+    counter = torch.zeros(len(cseg), dtype=torch.int32, device=dev)
+    RA = tiling.reorder_indices(T, hint, dev).reshape(TM, TN)
+    o = _overlap(api)
+    o.set_consumer_mode(mode)
+    g = torch.Generator().manual_seed(1)
+    W = (torch.randn(N, generator=g) * 0.5).to(torch.float16).to(dev)
+    cases = [(torch.ones(M, K, dtype=torch.float16), torch.ones(N, K, dtype=torch.float16)),
+             ((torch.randn(M, K, generator=g) / K ** 0.5).half(), (torch.randn(N, K, generator=g) / K ** 0.5).half())]
+    for A, B in cases:
+        C = torch.empty(M, N, dtype=torch.float16, device=dev)
+        o.gemm_allreduce_overlap(A.to(dev), B.to(dev), C, counter, RA, 1, cSeg_CPU, cSeg_GPU, algo, False)
+        y = torch.empty(M, N, dtype=torch.float16, device=dev)
+        torch.ops.flashoverlap_op.reorder_rmsnorm(o.staging().view(M, N), y, W, BM, BN, 1, RA)
+        torch.cuda.synchronize()
+        assert _timeouts() == 0
+        assert counter.cpu().sum() == 0
+        cref = O.gemm(A, B)
+        assert torch.equal(o.staging().cpu(), O.place_tiles(cref, RA.cpu().numpy(), BM, BN, 1)) or \
+            O.rel_l2(o.staging().cpu(), O.place_tiles(cref, RA.cpu().numpy(), BM, BN, 1)) < 1e-3
+        ref = O.rmsnorm(cref, W.cpu(), 1e-5)
+        assert torch.allclose(y.cpu().float(), ref.float(), atol=1e-2, rtol=1e-2)      # the reference's own bar
+        assert O.rel_l2(y.cpu(), ref) < 1e-3 and O.max_abs(y.cpu(), ref) < 2e-2
+
+
+@pytest.mark.parametrize("stacked", [False, True])
+def test_reducescatter_overlap_like_correctness_rs(api, dev, stacked):
+    """example/correctness_rs.py:100-142 with an emulated world of 4: rank k's
+    receive buffer, normalised with BM // world_size, equals RMSNorm of the
+    rows k, k+ws, ... of the product."""
+    M, N, K, algo, ws, rank = 1024, 512, 256, 1, 4, 2
+    BM, BN, _ = capi.algo_tile(algo)
+    TM, TN = M // BM, N // BN
+    T = TM * TN
+    hint = tiling.raster_hint(M, N, algo)
+    cseg = [5, 11, 16]
+    cSeg_CPU = torch.tensor(cseg, dtype=torch.int32)
+    cSeg_GPU = cSeg_CPU.to(dev)
+    counter = torch.zeros(TN, dtype=torch.int32, device=dev)
+    RA = tiling.reorder_indices(T, hint, dev).reshape(TM, TN)
+    RE = tiling.generate_row_remap_array(M, N, BM, BN, cseg, ws, dev)
+    g = torch.Generator().manual_seed(2)
+    A0 = (torch.randn(M, K, generator=g) * 0.5).to(torch.bfloat16)
+    B = (torch.randn(N, K, generator=g) * 0.5).to(torch.bfloat16)
+    W = (torch.randn(N, generator=g) * 0.5).to(torch.bfloat16)
+    o = _overlap(api, rank, ws)
+    tmp = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    out = torch.zeros((ws, M // ws, N) if stacked else (M // ws, N), dtype=torch.bfloat16, device=dev)
+    o.gemm_reducescatter_overlap(A0.to(dev), B.to(dev), tmp, out, counter, RA, RE, 1, cSeg_CPU, cSeg_GPU, algo, False)
+    torch.cuda.synchronize()
+    assert _timeouts() == 0 and counter.cpu().sum() == 0
+    cref = O.gemm(A0, B)
+    slices = O.consume_reducescatter(O.scatter_place(cref, RA.cpu().numpy(), RE.cpu().numpy(), BM, BN, 1), cseg, BM,
+                                     BN, ws)
+    mine = out[rank] if stacked else out
+    if stacked:
+        assert O.rel_l2(out.cpu().view(ws, -1), slices) < 1e-3
+    assert O.rel_l2(mine.cpu().view(-1), slices[rank]) < 1e-3
+    y = torch.empty(M // ws, N, dtype=torch.bfloat16, device=dev)
+    torch.ops.flashoverlap_op.reorder_rmsnorm(mine.contiguous(), y, W.to(dev), BM // ws, BN, 1, RA)
+    torch.cuda.synchronize()
+    x1 = O.reorder_rows_by_world_size(cref, ws).view(ws, M // ws, N)[rank]      # what the reference compares against
+    ref = O.rmsnorm(x1, W, 1e-5)
+    assert torch.allclose(y.cpu().float(), ref.float(), atol=5e-2, rtol=5e-2)     # the reference's own bar
+    assert O.rel_l2(y.cpu(), ref) < 2.5e-3  # bf16 output rounding of a storage-matched oracle, C itself may differ by an ulp
+
+
+def test_monitor_pass_like_the_tuner(api, dev):
+    # tune/search.py:164-187
+    M, N, K, algo = 2048, 2048, 128, 1
+    BM, BN, _ = capi.algo_tile(algo)
+    TM, TN = M // BM, N // BN
+    T = TM * TN
+    cseg = tiling.uniform_cseg(T, 100)
+    cSeg_CPU = torch.tensor(cseg, dtype=torch.int32)
+    MonitoredMatrix = torch.zeros((TM + 1, TN), dtype=torch.int32, device=dev)
+    ReorderedArray = torch.arange(0, T, dtype=torch.int32, device=dev).reshape(TM, TN)
+    A = torch.randn(M, K, dtype=torch.float16, device=dev)
+    B = torch.randn(N, K, dtype=torch.float16, device=dev)
+    C = torch.empty(M, N, dtype=torch.float16, device=dev)
+    o = _overlap(api)
+    samples = torch.empty((3, T), dtype=torch.int32, device=dev)
+    for i in range(3):
+        MonitoredMatrix[0] = 0
+        o.gemm_allreduce_overlap(A, B, C, MonitoredMatrix, ReorderedArray, 1, cSeg_CPU, cSeg_CPU.to(dev), algo, True)
+        samples[i, :] = MonitoredMatrix[1:, :].view(-1)
+    torch.cuda.synchronize()
+    assert _timeouts() == 0
+    for i in range(3):
+        assert sorted(samples[i].cpu().tolist()) == list(range(T))
+    assert MonitoredMatrix[0, TN - 1].item() == T
+
+
+def test_api_argument_checks(api, dev):
+    o = _overlap(api)
+    M = N = K = 256
+    A = torch.zeros(M, K, dtype=torch.float16, device=dev)
+    C = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    RA = torch.arange(4, dtype=torch.int32, device=dev).reshape(2, 2)
+    mm = torch.zeros(4, dtype=torch.int32, device=dev)
+    good = torch.tensor([4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="sum\\(cSeg\\)"):
+        bad = torch.tensor([3], dtype=torch.int32)
+        o.gemm_allreduce_overlap(A, A, C, mm, RA, 1, bad, bad.to(dev), 1, False)
+    with pytest.raises(RuntimeError, match="counters"):
+        many = torch.tensor([1, 1, 1, 1], dtype=torch.int32)
+        o.gemm_allreduce_overlap(A, A, C, mm[:2], RA, 1, many, many.to(dev), 1, False)
+    with pytest.raises(RuntimeError, match="RA is"):
+        o.gemm_allreduce_overlap(A, A, C, mm, RA.reshape(1, 4), 1, good, good.to(dev), 1, False)
+    with pytest.raises(RuntimeError, match="dtype"):
+        o.gemm_allreduce_overlap(A, A.bfloat16(), C, mm, RA, 1, good, good.to(dev), 1, False)
+    with pytest.raises(RuntimeError, match="Algo"):
+        o.mutlass_gemm(A, A, C, 17)
+    with pytest.raises(RuntimeError, match="more than one GPU"):
+        _overlap(api, 0, 2).gemm_all2all(A, A, C, C, 1, torch.zeros(2, 2, dtype=torch.int32))
+    torch.cuda.synchronize()
+    assert _timeouts() == 0

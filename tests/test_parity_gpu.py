@@ -1,0 +1,466 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU
+oracle on the same seeded inputs.
+
+Bars: integer artefacts (counters, tickets, group table, placement, staging,
+row remap) bit-exact; GEMM on small-integer inputs bit-exact (every partial sum
+is exact in fp32, so accumulation order cannot matter and any indexing mistake
+shows); GEMM + RMSNorm on random inputs within rel-L2 1e-3 and max-abs 2e-2 of
+the fp32 oracle cast through the same storage points (C -> dtype, out ->
+dtype); the distance to the unquantised fp32 result is printed as information.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from flashoverlap_amd import capi, tiling
+from oracle import fo_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL = 1e-3
+MAX_ABS_TOL = 2e-2
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+class Path:
+    """One problem instance with its device buffers, driven through the C ABI."""
+
+    def __init__(self, L, dev, dt, M, N, K, algo, cseg=None, hint=None, ws=1, monitor=False, seed=0,
+                 integer_inputs=False, a_std=None, b_std=None):
+        self.L, self.dev, self.dt = L, dev, dt
+        self.M, self.N, self.K, self.algo, self.ws, self.monitor = M, N, K, algo, ws, monitor
+        self.BM, self.BN, _ = capi.algo_tile(algo)
+        self.TM, self.TN = M // self.BM, N // self.BN
+        self.T = self.TM * self.TN
+        g = torch.Generator().manual_seed(seed)
+        if integer_inputs:
+            self.A = torch.randint(-2, 3, (M, K), generator=g).to(dt)
+            self.B = torch.randint(-2, 3, (N, K), generator=g).to(dt)
+        else:
+            sa = a_std if a_std is not None else 1.0 / K ** 0.5
+            sb = b_std if b_std is not None else 1.0 / K ** 0.5
+            self.A = (torch.randn(M, K, generator=g) * sa).to(dt)
+            self.B = (torch.randn(N, K, generator=g) * sb).to(dt)
+        self.gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(dt)
+        self.hint = list(hint) if hint is not None else tiling.raster_hint(M, N, algo)
+        self.cseg = list(cseg) if cseg is not None else [self.T]
+        self.G = len(self.cseg)
+        self.ra_host = tiling.reorder_indices(self.T, self.hint)
+        self.dA, self.dB, self.dgamma = self.A.to(dev), self.B.to(dev), self.gamma.to(dev)
+        self.dRA = self.ra_host.to(dev).reshape(self.TM, self.TN)
+        self.dcseg = torch.tensor(self.cseg, dtype=torch.int32, device=dev)
+        mm_len = (self.TN + self.T) if monitor else max(self.G, self.TN)
+        self.dMM = torch.zeros(mm_len, dtype=torch.int32, device=dev)
+        self.dtable = torch.full((self.T,), -1, dtype=torch.int32, device=dev)
+        self.dC = torch.zeros(M * N, dtype=dt, device=dev)
+        self.re_host = None
+        self.dRE = None
+        if ws > 1:
+            self.re_host = tiling.generate_row_remap_array(M, N, self.BM, self.BN, self.cseg, ws)
+            self.dRE = self.re_host.to(dev)
+        self.code = capi.dtype_code(dt)
+
+    def build_table(self, stream=None):
+        capi.check(self.L.fo_build_group_table(self.dcseg.data_ptr(), self.G, self.T, self.dtable.data_ptr(), stream))
+
+    def gemm_plain(self, out=None, stream=None):
+        out = out if out is not None else torch.zeros(self.M, self.N, dtype=self.dt, device=self.dev)
+        capi.check(self.L.fo_gemm(self.code, self.algo, self.M, self.N, self.K, self.dA.data_ptr(),
+                                  self.dB.data_ptr(), out.data_ptr(), stream))
+        return out
+
+    def gemm_signal(self, use_table=True, stream=None):
+        table = self.dtable.data_ptr() if use_table else None
+        if self.ws > 1:
+            capi.check(self.L.fo_gemm_scatter(self.code, self.algo, self.M, self.N, self.K, 1, self.dcseg.data_ptr(),
+                                              self.G, table, self.dA.data_ptr(), self.dB.data_ptr(),
+                                              self.dC.data_ptr(), self.dMM.data_ptr(), self.dRA.data_ptr(),
+                                              self.dRE.data_ptr(), int(self.monitor), stream))
+        else:
+            capi.check(self.L.fo_gemm_signal(self.code, self.algo, self.M, self.N, self.K, 1, self.dcseg.data_ptr(),
+                                             self.G, table, self.dA.data_ptr(), self.dB.data_ptr(),
+                                             self.dC.data_ptr(), self.dMM.data_ptr(), self.dRA.data_ptr(),
+                                             int(self.monitor), stream))
+
+    def reorder_rmsnorm(self, x, eps, bs=None, BM=None, stream=None):
+        bs = bs if bs is not None else self.M
+        BM = BM if BM is not None else self.BM
+        out = torch.empty(bs, self.N, dtype=self.dt, device=self.dev)
+        capi.check(self.L.fo_reorder_rmsnorm(self.code, x.data_ptr(), self.dgamma.data_ptr(), out.data_ptr(), bs,
+                                             self.N, BM, self.BN, 1, self.dRA.data_ptr(), eps, stream))
+        return out
+
+
+@pytest.fixture(scope="module")
+def L(fo_lib, dev):
+    capi.check(fo_lib.fo_set_wait_timeout_ms(5000))
+    return fo_lib
+
+
+@pytest.fixture()
+def comm_stream(L):
+    s = C.c_void_p()
+    capi.check(L.fo_stream_create(C.byref(s)))
+    yield s
+    capi.check(L.fo_stream_sync(s))
+    capi.check(L.fo_stream_destroy(s))
+
+
+def _timeouts(L):
+    n = C.c_int()
+    capi.check(L.fo_wait_timeouts(C.byref(n), 1))
+    return n.value
+
+
+# ---- GEMM --------------------------------------------------------------------
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K,algo", [(128, 128, 64, 1), (256, 256, 64, 0), (256, 512, 192, 3), (512, 256, 128, 5),
+                                        (384, 640, 320, 1), (1024, 1024, 1024, 1), (2048, 4096, 256, 1)])
+def test_gemm_bit_exact_on_integer_inputs(L, dev, dt, M, N, K, algo):
+    _say("gemm integer", dt, M, N, K, algo)
+    p = Path(L, dev, dt, M, N, K, algo, integer_inputs=True)
+    got = p.gemm_plain()
+    torch.cuda.synchronize()
+    want = O.gemm(p.A, p.B)
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_gemm_random_within_tolerance(L, dev, dt):
+    M, N, K = 1024, 768, 2048
+    _say("gemm random", dt, M, N, K)
+    p = Path(L, dev, dt, M, N, K, 1, seed=3)
+    got = p.gemm_plain().cpu()
+    ref32 = O.gemm_fp32(p.A, p.B)
+    gated = ref32.to(dt)
+    _say("  vs unquantised fp32: rel-L2 %.2e max-abs %.2e" % (O.rel_l2(got, ref32), O.max_abs(got, ref32)))
+    assert O.rel_l2(got, gated) < REL_L2_TOL and O.max_abs(got, gated) < MAX_ABS_TOL
+    # fp32 accumulation order is the only freedom: at most one storage ulp apart
+    ulp = 2 ** -10 if dt == torch.float16 else 2 ** -7
+    assert ((got.float() - gated.float()).abs() <= ulp * gated.float().abs() + 1e-6).all()
+
+
+def test_gemm_rejects_unsupported_shapes(L, dev):
+    a = torch.zeros(256, 96, dtype=torch.float16, device=dev)
+    assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 96, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
+    assert L.fo_gemm(capi.FO_F16, 3, 384, 384, 64, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
+
+
+# ---- signalling epilogue -------------------------------------------------------
+
+@pytest.mark.parametrize("dt,M,N,K,algo,w", [
+    (torch.float16, 1024, 1024, 1024, 1, 4),      # BASELINE config 1: 64 tiles, 16 groups of 4 (> TN = 8 counters)
+    (torch.bfloat16, 512, 768, 128, 1, 5),        # ragged last group
+    (torch.float16, 1024, 2048, 64, 3, 3),        # 128x256 layout tile
+    (torch.bfloat16, 2048, 1024, 64, 5, 7),       # 256x128 layout tile
+    (torch.float16, 2048, 2048, 64, 1, 1),        # one tile per group: 256 counters
+])
+def test_signal_placement_counters_and_table(L, dev, dt, M, N, K, algo, w):
+    _say("signal", dt, M, N, K, algo, w)
+    BM, BN, _ = capi.algo_tile(algo)
+    T = (M // BM) * (N // BN)
+    rng = np.random.default_rng(5)
+    hint = rng.permutation(T).tolist()  # any permutation is legal, not only the raster order
+    p = Path(L, dev, dt, M, N, K, algo, cseg=O.uniform_cseg(T, w), hint=hint, integer_inputs=True)
+    p.build_table()
+    torch.cuda.synchronize()
+    assert p.dtable.cpu().tolist() == O.group_of_slots(p.cseg, range(T)).tolist()
+    assert p.ra_host.tolist() == O.reorder_indices(T, hint).tolist()
+
+    natural = p.gemm_plain()
+    p.gemm_signal()
+    torch.cuda.synchronize()
+    # counters: every group has seen exactly its tiles
+    assert p.dMM.cpu()[:p.G].tolist() == p.cseg
+    assert p.dMM.cpu()[p.G:].sum() == 0
+    # placement: bit-exact against the oracle's epilogue applied to the natural GEMM, and to the oracle GEMM
+    assert torch.equal(p.dC.cpu(), O.place_tiles(natural.cpu(), p.ra_host.numpy(), BM, BN, 1))
+    assert torch.equal(p.dC.cpu(), O.place_tiles(O.gemm(p.A, p.B), p.ra_host.numpy(), BM, BN, 1))
+    # same result with the reference's in-kernel linear scan instead of the table
+    p.dMM.zero_()
+    p.dC.zero_()
+    p.gemm_signal(use_table=False)
+    torch.cuda.synchronize()
+    assert p.dMM.cpu()[:p.G].tolist() == p.cseg
+    assert torch.equal(p.dC.cpu(), O.place_tiles(natural.cpu(), p.ra_host.numpy(), BM, BN, 1))
+
+
+def test_group_table_edge_cases(L, dev):
+    for cseg, T in (([5], 5), ([1] * 300, 300), ([0, 3, 0, 0, 2, 1], 6), ([2000, 48], 2048), ([3, 3], 8)):
+        d = torch.tensor(cseg, dtype=torch.int32, device=dev)
+        table = torch.full((T,), -7, dtype=torch.int32, device=dev)
+        capi.check(L.fo_build_group_table(d.data_ptr(), len(cseg), T, table.data_ptr(), None))
+        torch.cuda.synchronize()
+        covered = min(T, sum(cseg))
+        assert table.cpu()[:covered].tolist() == O.group_of_slots(cseg, range(covered)).tolist()
+        assert (table.cpu()[covered:] == len(cseg) - 1).all()  # beyond sum(cSeg): clamped, stays in bounds
+
+
+def test_monitor_mode_tickets(L, dev):
+    # tune/search.py:164-187: identity RA, MM of (TM+1) x TN, tickets in MM[1:, :]
+    M = N = 2048
+    K = 64
+    BM = BN = 128
+    T = 256
+    TN = N // BN
+    cseg = O.uniform_cseg(T, 64)
+    p = Path(L, dev, torch.float16, M, N, K, 1, cseg=cseg, hint=list(range(T)), monitor=True, integer_inputs=True)
+    p.build_table()
+    p.gemm_signal()
+    torch.cuda.synchronize()
+    mm = p.dMM.cpu()
+    tickets = mm[TN:].tolist()
+    assert sorted(tickets) == list(range(T))          # a permutation of 0..T-1
+    assert mm[TN - 1] == T                            # the ticket counter
+    assert mm[:len(cseg)].tolist() == cseg            # group counters untouched by the tickets
+
+
+@pytest.mark.parametrize("ws,cseg_w", [(2, 3), (8, 4), (4, 16)])
+def test_scatter_epilogue_and_reducescatter_slices(L, dev, comm_stream, ws, cseg_w):
+    M, N, K, algo = 1024, 512, 128, 1
+    _say("scatter", ws, cseg_w)
+    BM, BN, _ = capi.algo_tile(algo)
+    T = (M // BM) * (N // BN)
+    cseg = O.uniform_cseg(T, cseg_w)
+    p = Path(L, dev, torch.bfloat16, M, N, K, algo, cseg=cseg, ws=ws, integer_inputs=True, seed=7)
+    assert p.re_host.tolist() == O.row_remap(M, N, BM, BN, cseg, ws).tolist()
+    p.build_table()
+    p.gemm_signal()
+    torch.cuda.synchronize()
+    natural = O.gemm(p.A, p.B)
+    want = O.scatter_place(natural, p.ra_host.numpy(), p.re_host.numpy(), BM, BN, 1)
+    assert torch.equal(p.dC.cpu(), want)
+    assert p.dMM.cpu()[:p.G].tolist() == cseg
+    # consumer: all ws receive buffers side by side
+    D = torch.zeros(ws, M * N // ws, dtype=p.dt, device=dev)
+    capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), D.data_ptr(), BM * BN,
+                                 ws, 0, ws, M * N // ws, None, 4, comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert _timeouts(L) == 0
+    assert torch.equal(D.cpu(), O.consume_reducescatter(want, cseg, BM, BN, ws))
+    assert p.dMM.cpu().sum() == 0
+    # each slice is a permuted layout with tile height BM/ws of the rows m % ws == k;
+    # reorder+RMSNorm with BM/ws on it equals RMSNorm of those rows
+    for k in (0, ws - 1):
+        out = p.reorder_rmsnorm(D[k], 1e-5, bs=M // ws, BM=BM // ws)
+        torch.cuda.synchronize()
+        ref = O.rmsnorm(natural[k::ws], p.gamma, 1e-5)
+        assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and O.max_abs(out.cpu(), ref) < MAX_ABS_TOL
+    # one rank's view: only slice 1
+    p.gemm_signal()
+    one = torch.zeros(M * N // ws, dtype=p.dt, device=dev)
+    capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), one.data_ptr(), BM * BN,
+                                 ws, 1, 1, 0, None, 2, comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert torch.equal(one.cpu(), O.consume_reducescatter(want, cseg, BM, BN, ws)[1])
+
+
+# ---- wait / consume ------------------------------------------------------------
+
+def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
+    mm = torch.tensor([3, 9], dtype=torch.int32, device=dev)
+    capi.check(L.fo_wait(3, mm.data_ptr(), comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert mm.cpu().tolist() == [0, 9] and _timeouts(L) == 0
+    # a count that is never reached: the waiter gives up after the limit, leaves
+    # the counter alone and the stream carries on (the reference would spin forever)
+    capi.check(L.fo_set_wait_timeout_ms(50))
+    try:
+        capi.check(L.fo_wait(5, mm.data_ptr() + 4, comm_stream))
+        capi.check(L.fo_stream_sync(comm_stream))
+        assert mm.cpu().tolist() == [0, 9] and _timeouts(L) == 1
+        src = torch.arange(4096, dtype=torch.int16, device=dev)
+        dst = torch.zeros_like(src)
+        bad = torch.tensor([1, 1], dtype=torch.int32, device=dev)
+        flags = torch.tensor([1, 0], dtype=torch.int32, device=dev)   # group 1 never completes
+        capi.check(L.fo_wait_consume(bad.data_ptr(), 2, flags.data_ptr(), src.data_ptr(), dst.data_ptr(), 2048, 1, 0,
+                                     1, 0, None, 3, comm_stream))
+        capi.check(L.fo_stream_sync(comm_stream))
+        assert _timeouts(L) == 3                      # every workgroup reports and leaves
+        assert torch.equal(dst[:2048], src[:2048]) and not dst[2048:].any()
+    finally:
+        capi.check(L.fo_set_wait_timeout_ms(5000))
+
+
+def test_consume_copies_exactly_the_bytes(L, dev):
+    src = torch.randint(-30000, 30000, (100003,), dtype=torch.int16, device=dev)
+    for off, n in ((0, 100003), (8, 77), (16, 8), (24, 4099)):
+        dst = torch.full_like(src, -1)
+        capi.check(L.fo_consume(src.data_ptr() + 2 * off, dst.data_ptr() + 2 * off, 2 * n, None))
+        torch.cuda.synchronize()
+        assert torch.equal(dst[off:off + n], src[off:off + n])
+        assert (dst[:off] == -1).all() and (dst[off + n:] == -1).all()
+
+
+@pytest.mark.parametrize("mode", ["per_group", "persistent"])
+def test_overlapped_release_order_and_staging(L, dev, comm_stream, mode):
+    """GEMM on one stream, waiter/consumer on another, started together; run
+    twice with different A so that a stale cache line in the consumer would show."""
+    M, N, K, algo = 2048, 2048, 512, 1
+    BM, BN, _ = capi.algo_tile(algo)
+    T = 256
+    cseg = [40, 24, 64, 1, 127]
+    _say("overlap", mode)
+    p = Path(L, dev, torch.float16, M, N, K, algo, cseg=cseg, integer_inputs=True, seed=11)
+    p.build_table()
+    staging = torch.zeros(M * N, dtype=p.dt, device=dev)
+    log = torch.full((p.G,), -1, dtype=torch.int32, device=dev)
+    for rep in range(2):
+        if rep == 1:
+            p.A = -p.A
+            p.dA = p.A.to(dev)
+        staging.zero_()
+        torch.cuda.synchronize()
+        p.gemm_signal()
+        if mode == "persistent":
+            capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(),
+                                         staging.data_ptr(), BM * BN, 1, 0, 1, 0, log.data_ptr(), 6, comm_stream))
+        else:
+            acc = 0
+            for g, n in enumerate(cseg):
+                capi.check(L.fo_wait(n, p.dMM.data_ptr() + 4 * g, comm_stream))
+                capi.check(L.fo_consume(p.dC.data_ptr() + 2 * acc, staging.data_ptr() + 2 * acc, 2 * n * BM * BN,
+                                        comm_stream))
+                acc += n * BM * BN
+        capi.check(L.fo_stream_join(comm_stream, None))
+        torch.cuda.synchronize()
+        assert _timeouts(L) == 0
+        want = O.place_tiles(O.gemm(p.A, p.B), p.ra_host.numpy(), BM, BN, 1)
+        assert torch.equal(p.dC.cpu(), want)
+        assert torch.equal(staging.cpu(), O.consume_allreduce(want, cseg, BM, BN))
+        assert p.dMM.cpu().sum() == 0                     # every counter back to zero for the next call
+        if mode == "persistent":
+            assert log.cpu().tolist() == list(range(p.G))  # released in index order
+
+
+# ---- RMSNorm -------------------------------------------------------------------
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bs,dim", [(4, 8), (7, 520), (33, 1024), (16, 4096), (5, 8192), (3, 16384), (9, 4104)])
+def test_plain_rmsnorm(L, dev, dt, bs, dim):
+    g = torch.Generator().manual_seed(bs * dim)
+    x = torch.randn(bs, dim, generator=g).to(dt)
+    gamma = (1 + 0.1 * torch.randn(dim, generator=g)).to(dt)
+    out = torch.empty(bs, dim, dtype=dt, device=dev)
+    dx, dgamma = x.to(dev), gamma.to(dev)
+    capi.check(L.fo_rmsnorm(capi.dtype_code(dt), dx.data_ptr(), dgamma.data_ptr(), out.data_ptr(), bs, dim, 1e-5, None))
+    torch.cuda.synchronize()
+    ref = O.rmsnorm(x, gamma, 1e-5)
+    assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and O.max_abs(out.cpu(), ref) < MAX_ABS_TOL
+    # same two-rounding order as the reference kernel: within two storage ulps of the oracle
+    ulp = 2 ** -10 if dt == torch.float16 else 2 ** -7
+    assert ((out.cpu().float() - ref.float()).abs() <= 2 * ulp * ref.float().abs() + 1e-6).all()
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bs,dim,BM,BN,rldn", [(256, 512, 128, 128, 1), (256, 512, 128, 128, 2), (128, 1024, 64, 256, 1),
+                                               (64, 384, 16, 8, 1), (96, 4096, 32, 128, 1)])
+def test_reorder_rmsnorm(L, dev, dt, bs, dim, BM, BN, rldn):
+    g = torch.Generator().manual_seed(dim + BM)
+    Cn = torch.randn(bs, dim, generator=g).to(dt)
+    gamma = (1 + 0.1 * torch.randn(dim, generator=g)).to(dt)
+    T = (bs // BM) * (dim // BN)
+    ra = O.reorder_indices(T, np.random.default_rng(T).permutation(T))
+    x = O.place_tiles(Cn, ra, BM, BN, rldn)
+    out = torch.empty(bs, dim, dtype=dt, device=dev)
+    dx, dgamma, dra = x.to(dev), gamma.to(dev), torch.from_numpy(ra).to(dev)
+    capi.check(L.fo_reorder_rmsnorm(capi.dtype_code(dt), dx.data_ptr(), dgamma.data_ptr(), out.data_ptr(), bs, dim,
+                                    BM, BN, rldn, dra.data_ptr(), 1e-6, None))
+    torch.cuda.synchronize()
+    ref = O.reorder_rmsnorm(x, gamma, bs, dim, BM, BN, rldn, ra, 1e-6)
+    assert torch.equal(ref, O.rmsnorm(Cn, gamma, 1e-6))
+    assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and O.max_abs(out.cpu(), ref) < MAX_ABS_TOL
+    # eps really is a parameter: a large one changes the result the way the formula says
+    capi.check(L.fo_reorder_rmsnorm(capi.dtype_code(dt), dx.data_ptr(), dgamma.data_ptr(), out.data_ptr(), bs, dim,
+                                    BM, BN, rldn, dra.data_ptr(), 3.0, None))
+    torch.cuda.synchronize()
+    ref3 = O.rmsnorm(Cn, gamma, 3.0)
+    assert O.rel_l2(out.cpu(), ref3) < REL_L2_TOL
+
+
+# ---- BASELINE configurations, full size ------------------------------------------
+
+def _full_path(L, dev, comm_stream, dt, M, N, K, w, eps, ws=1, a_std=None, b_std=None, check_rows=None):
+    """Whole hot path on random inputs at full size: signalling GEMM overlapped
+    with the persistent consumer, then reorder+RMSNorm, against the oracle."""
+    algo = 1
+    BM, BN, _ = capi.algo_tile(algo)
+    T = (M // BM) * (N // BN)
+    cseg = O.uniform_cseg(T, w)
+    p = Path(L, dev, dt, M, N, K, algo, cseg=cseg, ws=ws, a_std=a_std, b_std=b_std)
+    p.build_table()
+    dst = torch.zeros(M * N, dtype=dt, device=dev)
+    p.gemm_signal()
+    capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), dst.data_ptr(), BM * BN,
+                                 ws, 0, ws, M * N // ws if ws > 1 else 0, None, 8, comm_stream))
+    capi.check(L.fo_stream_join(comm_stream, None))
+    torch.cuda.synchronize()
+    assert _timeouts(L) == 0
+    assert p.dMM.cpu().sum() == 0
+    if ws == 1:
+        assert torch.equal(dst, p.dC)                      # staging is the permuted C, bit for bit
+        out = p.reorder_rmsnorm(dst, eps)
+        torch.cuda.synchronize()
+        rows = torch.arange(M) if check_rows is None else check_rows
+        got = out.cpu()[rows]
+        src_rows = rows
+    else:
+        # every slice k holds the rows m % ws == k as a layout with tile height BM/ws
+        outs = [p.reorder_rmsnorm(dst.view(ws, -1)[k], eps, bs=M // ws, BM=BM // ws) for k in range(ws)]
+        torch.cuda.synchronize()
+        full = torch.empty(M, N, dtype=dt)
+        for k in range(ws):
+            full[k::ws] = outs[k].cpu()
+        rows = torch.arange(M) if check_rows is None else check_rows
+        got = full[rows]
+        src_rows = rows
+    c32 = O.gemm_fp32(p.A[src_rows], p.B)
+    gated = O.rmsnorm(c32.to(dt), p.gamma, eps)
+    unq = O.rmsnorm_fp32(c32, p.gamma, eps)
+    _say("  vs unquantised fp32: rel-L2 %.2e max-abs %.2e" % (O.rel_l2(got, unq), O.max_abs(got, unq)))
+    _say("  vs storage-matched : rel-L2 %.2e max-abs %.2e" % (O.rel_l2(got, gated), O.max_abs(got, gated)))
+    assert O.rel_l2(got, gated) < REL_L2_TOL and O.max_abs(got, gated) < MAX_ABS_TOL
+    # permutation invariants at full size: un-permuting the signalled output gives the plain kernel's output
+    natural = p.gemm_plain()
+    torch.cuda.synchronize()
+    if ws == 1:
+        back = p.dC.view(T, BM, BN)[p.dRA.view(-1).long()].view(p.TM, p.TN, BM, BN).permute(0, 2, 1, 3).reshape(M, N)
+        assert torch.equal(back, natural)
+    return p
+
+
+def test_config1_fp16_1024(L, dev, comm_stream):
+    _say("config 1")
+    _full_path(L, dev, comm_stream, torch.float16, 1024, 1024, 1024, 4, 1e-6)
+
+
+@pytest.mark.parametrize("w", [1, 2, 4, 8, 16])
+def test_config2_fp16_4096_group_sweep(L, dev, comm_stream, w):
+    _say("config 2, group size", w)
+    rows = torch.arange(0, 4096, 37)
+    _full_path(L, dev, comm_stream, torch.float16, 4096, 4096, 4096, w, 1e-5, check_rows=rows)
+
+
+def test_config3_bf16_llama8b_down_proj(L, dev, comm_stream):
+    _say("config 3")
+    rows = torch.arange(0, 8192, 61)
+    _full_path(L, dev, comm_stream, torch.bfloat16, 8192, 4096, 7168, 256, 1e-5, a_std=1.0, b_std=0.02,
+               check_rows=rows)
+
+
+def test_config4_bf16_small_k_many_groups(L, dev, comm_stream):
+    _say("config 4")
+    rows = torch.arange(0, 16384, 251)
+    _full_path(L, dev, comm_stream, torch.bfloat16, 16384, 8192, 1024, 2, 1e-5, check_rows=rows)
+
+
+def test_config5_bf16_reducescatter_layout(L, dev, comm_stream):
+    _say("config 5")
+    rows = torch.arange(0, 8192, 127)
+    _full_path(L, dev, comm_stream, torch.bfloat16, 8192, 8192, 3584, 256, 1e-5, ws=8, check_rows=rows)
