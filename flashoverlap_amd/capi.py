@@ -28,6 +28,7 @@ SIGNATURES = {
     "fo_gemm_scatter": (_i, [_i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "fo_build_group_table": (_i, [_vp, _i, _i, _vp, _vp]),
     "fo_raster_hint": (_i, [_i, _i, _i, _ip]),
+    "fo_tune": (_i, [C.c_char_p, _i]),
     "fo_wait": (_i, [_i, _vp, _vp]),
     "fo_wait_consume": (_i, [_vp, _i, _vp, _vp, _vp, _ll, _i, _i, _i, _ll, _vp, _i, _vp]),
     "fo_set_wait_timeout_ms": (_i, [_i]),

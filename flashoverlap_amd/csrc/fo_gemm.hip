@@ -3,23 +3,33 @@
 //
 // One workgroup of 4 wavefronts computes one MT x MT macro tile (MT = 256, or
 // 128 for small problems); each wavefront owns an (MT/2) x (MT/2) quadrant as
-// (MT/64)^2 blocks of v_mfma_f32_32x32x16.  A and B panels of 64 k-elements
-// are streamed HBM -> LDS with global_load_lds_dwordx4 (no register staging)
-// into two LDS stages; the 16-byte chunks of a row are XOR-swizzled by row so
-// that the ds_read_b128 fragment reads are bank-conflict free.
+// (MT/64)^2 blocks of v_mfma_f32_32x32x16, accumulators in AGPRs.
 //
-// The epilogue writes the quadrant either to the natural row-major D (plain
-// GEMM) or to the slot RA[tile] of the tile-permuted layout, optionally with
-// the row index mapped through RE (scatter), and then signals: after every
-// wavefront's stores have been acknowledged and the workgroup has met at a
-// barrier, one lane per layout tile bumps the tile's group counter with a
-// release-ordered, agent-scope atomic.  The plain GEMM is the same kernel
-// instantiated with the signalling code compiled out.
+// Main loop: A and B panels of 32 k-elements stream HBM -> LDS with
+// global_load_lds_dwordx4 (no register staging) through a ring of 4 LDS
+// stages, so copies are issued three k-steps ahead of their use.  The 16-byte
+// chunks of a tile row are XOR-swizzled by row so the ds_read_b128 fragment
+// reads are bank-conflict free.  Fragments are double-buffered in registers:
+// while the 16 MFMAs of one half k-step run, the fragments of the next half
+// step (possibly of the next stage) are already being read, and there is one
+// workgroup barrier per k-step.
+//
+// Epilogue: the quadrant goes through LDS in strips of 32 rows so that every
+// global store instruction writes four whole 256-byte row segments, either to
+// the natural row-major D (plain GEMM) or to slot RA[tile] of the
+// tile-permuted layout, optionally with the row index mapped through RE
+// (scatter).  Then the signal: after every wavefront's stores have been
+// acknowledged and the workgroup has met at a barrier, one lane per layout
+// tile bumps the tile's group counter with a release-ordered, agent-scope
+// atomic.  The plain GEMM is the same kernel with the signalling compiled out.
 //
 // Semantics follow the reference epilogues src/overlap/gemm_with_signal.h:145-201
 // and src/overlap/gemm_with_scatter.h:146-196; the kernel itself shares nothing
 // with the reference's MUTlass mainloop.
 #include <hip/hip_runtime.h>
+
+#include <string_view>
+#include <type_traits>
 
 #include "fo_internal.h"
 #include "fo_raster.h"
@@ -31,6 +41,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T>
 struct Mma;
@@ -51,10 +62,16 @@ struct Mma<__bf16> {
     }
 };
 
-constexpr int kBK = 64;            // k-elements per LDS stage
-constexpr int kRowBytes = kBK * 2; // one tile row in LDS: 128 bytes = 8 chunks of 16
+constexpr int kBK = 32;             // k-elements per LDS stage
+constexpr int kRowBytes = kBK * 2;  // one tile row in LDS: 64 bytes = 4 chunks of 16
 
 enum { kPlain = 0, kSignal = 1, kScatter = 2 };
+
+// Tuning knobs (fo_tune): how the epilogue stores C and how it signals.
+int g_store_mode = 0;    // 0 = cached stores, 1 = agent-scope write-through stores (sc1)
+int g_release_mode = 0;  // 0 = release-ordered atomic, 1 = write-through stores + relaxed atomic (needs store mode 1)
+int g_stages = 4;        // LDS ring stages of the 256 macro tile (3, 4 or 5)
+int g_debug = 0;         // what-if timing variants of the bf16 256 plain kernel (wrong results)
 
 struct GemmParams {
     const void* A;
@@ -75,12 +92,17 @@ struct GemmParams {
 };
 
 typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((address_space(1))) const void gbl_void;
 
-// One 1 KiB wave-wide copy HBM -> LDS: lane l's 16 bytes land at lds + 16*l.
-__device__ __forceinline__ void async_copy16(const void* g, void* lds_wave_base) {
-    __builtin_amdgcn_global_load_lds((gbl_void*)g, (lds_void*)lds_wave_base, 16, 0, 0);
+// s_waitcnt immediate of the gfx9 family: vmcnt in bits [3:0] and [15:14],
+// expcnt [6:4], lgkmcnt [11:8]; 63 / 7 / 15 mean "do not wait".
+constexpr int waitcnt_imm(int vm, int lgkm) {
+    return (vm & 0xF) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm & 0xF) << 8);
 }
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(N, 15));
+}
+__device__ __forceinline__ void wait_lds_reads() { __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0)); }
 
 // The reference's linear scan over cSeg (src/overlap/gemm_with_signal.h:188-193).
 __device__ __forceinline__ int scan_group(const int* cseg, int slot) {
@@ -93,13 +115,36 @@ __device__ __forceinline__ int scan_group(const int* cseg, int slot) {
     return g;
 }
 
-template <typename T, int MT, int MODE>
+// Row swizzle shared by the copy and the fragment reads: LDS chunk (row, cc)
+// holds k-chunk cc ^ swz(row).  Conflict free for 8 or 16 consecutive rows.
+__device__ __forceinline__ int swz(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+
+template <int N>
+using template_int = std::integral_constant<int, N>;
+
+// f(integral_constant<0>) ... f(integral_constant<N-1>)
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(template_int<N - 1>{});
+    }
+}
+
+// STORE: 0 cached, 1 write-through tile stores; REL: 0 release atomic, 1 relaxed atomic;
+// NS: LDS ring stages; DBG: what-if timing variants that compute wrong results
+// (1 = no HBM->LDS copies in the main loop, 2 = no LDS fragment reads in the main loop,
+// 3 = every copy re-reads tile 0, 4 = no wait for the copies, 5 = no barrier in the main loop,
+// 6 = every copy re-reads the same 2 KiB, 7 = copies fetch whole 128-byte lines).
+template <typename T, int MT, int MODE, int STORE, int REL, int NS, int DBG>
 __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
-    constexpr int WT = MT / 2;          // wave quadrant edge
-    constexpr int NB = WT / 32;         // 32x32 MFMA blocks per quadrant edge
-    constexpr int PANEL = MT * kRowBytes;   // bytes of one A (or B) panel per stage
+    constexpr int WT = MT / 2;               // wave quadrant edge
+    constexpr int NB = WT / 32;              // 32x32 MFMA blocks per quadrant edge
+    constexpr int PANEL = MT * kRowBytes;    // bytes of one A (or B) panel per stage
     constexpr int STAGE = 2 * PANEL;
-    constexpr int LOADS = MT / 32;      // wave-wide 1 KiB copies per wave per panel
+    constexpr int LOADS = MT / 64;           // wave-wide 1 KiB copies per wave per panel
+    constexpr int LPT = 2 * LOADS;           // copies per wave per k-step
+    constexpr int BLK = 32 * kRowBytes;      // LDS bytes between 32-row blocks
     using frag = typename Mma<T>::frag;
     using out4 = typename Mma<T>::out4;
 
@@ -142,35 +187,45 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     }
 
     // ---- global -> LDS copy addressing ---------------------------------------
-    // A wave-wide copy fills 64 consecutive 16-byte LDS chunks = 8 tile rows.
-    // LDS chunk (row, cc) holds k-chunk cc ^ (row % 8) of that row.
-    const int cp_row = lane >> 3;                      // row within the 8-row slab
-    const int cp_kc = (lane & 7) ^ cp_row;             // k-chunk this lane fetches
-    const T* gA = (const T*)p.A + (size_t)(mt.m * MT + wave * (LOADS * 8) + cp_row) * K + cp_kc * 8;
-    const T* gB = (const T*)p.B + (size_t)(mt.n * MT + wave * (LOADS * 8) + cp_row) * K + cp_kc * 8;
-    const size_t slab_stride = (size_t)8 * K;          // elements between consecutive slabs
-    const int lds_cp = wave * (LOADS * 1024);          // this wave's first slab in a panel
+    // A wave-wide copy fills 64 consecutive 16-byte LDS chunks = 16 tile rows.
+    const int cp_row = lane >> 2;                      // row within the 16-row slab
+    const int cp_kc = (lane & 3) ^ swz(cp_row);        // k-chunk this lane fetches
+    // Buffer addressing: the operand is the buffer, the wave-uniform part of the
+    // offset (tile row, slab, k) lives in a scalar register and only the constant
+    // per-lane part in a vector register, so a copy costs no vector ALU work.
+    const int cp_off = DBG == 7 ? ((lane >> 3) * K + (lane & 7) * 8) * 2   // what-if: 8 rows x 128 B per copy
+                                : (cp_row * K + cp_kc * 8) * 2;
+    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, 0xffffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, 0xffffffff, 0x00020000);
+    const unsigned baseA = (unsigned)(mt.m * MT + wave * (LOADS * 16)) * (unsigned)K * 2u;
+    const unsigned baseB = (unsigned)(mt.n * MT + wave * (LOADS * 16)) * (unsigned)K * 2u;
+    const unsigned slab_bytes = 16u * (unsigned)K * 2u;   // bytes between consecutive slabs
+    const int lds_cp = wave * (LOADS * 1024);             // this wave's first slab in a panel
 
-    auto issue_loads = [&](int kt, int stage) {
-        unsigned char* sA = smem + stage * STAGE + lds_cp;
+    // Stage `st` of the ring receives tile `kt`; the copies of a tile are issued
+    // in two halves so that they can be spread over a whole k-step.  One copy
+    // moves 1 KiB: lane l's 16 bytes land at the LDS address + 16*l.
+    auto issue_half = [&](int kt, int st, auto half_c) {
+        constexpr int H = decltype(half_c)::value;
+        unsigned char* sA = smem + st * STAGE + lds_cp;
         unsigned char* sB = sA + PANEL;
-        const T* a = gA + (size_t)kt * kBK;
-        const T* b = gB + (size_t)kt * kBK;
+        const unsigned koff = (unsigned)(DBG == 3 ? 0 : kt) * (DBG == 7 ? 128 : kBK * 2) % (unsigned)(K * 2);
 #pragma unroll
-        for (int j = 0; j < LOADS; ++j) {
-            async_copy16(a + j * slab_stride, sA + j * 1024);
-            async_copy16(b + j * slab_stride, sB + j * 1024);
+        for (int j = H * (LOADS / 2); j < (H + 1) * (LOADS / 2); ++j) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(sA + j * 1024), 16, cp_off,
+                                                     (int)(baseA + (DBG == 6 ? 0 : j * slab_bytes + koff)), 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(sB + j * 1024), 16, cp_off,
+                                                     (int)(baseB + (DBG == 6 ? 0 : j * slab_bytes + koff)), 0, 0);
         }
     };
 
     // ---- LDS -> register fragment addressing ----------------------------------
     // MFMA 32x32x16 operand: lane l supplies row l%32, k = 8*(l/32) .. +7.
-    const int fr_row = lane & 31, fr_h = lane >> 5, fr_x = lane & 7;
+    const int fr_row = lane & 31, fr_h = lane >> 5;
     const int a_lane = (wm * WT + fr_row) * kRowBytes;
     const int b_lane = PANEL + (wn * WT + fr_row) * kRowBytes;
-    int ko[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) ko[kk] = ((2 * kk + fr_h) ^ fr_x) * 16;
+    const int ko0 = ((0 + fr_h) ^ swz(fr_row)) * 16;   // first half k-step (k 0..15)
+    const int ko1 = ((2 + fr_h) ^ swz(fr_row)) * 16;   // second half (k 16..31)
 
     f32x16 acc[NB][NB];
 #pragma unroll
@@ -180,39 +235,148 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    const int KT = K / kBK;
-    issue_loads(0, 0);
-    for (int kt = 0; kt < KT; ++kt) {
-        // Tile kt has landed for every wave, and every wave is done reading the
-        // stage that the next copies overwrite.
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (kt + 1 < KT) issue_loads(kt + 1, (kt + 1) & 1);
-        const unsigned char* st = smem + (kt & 1) * STAGE;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            frag a[NB], b[NB];
-#pragma unroll
-            for (int i = 0; i < NB; ++i) a[i] = *(const frag*)(st + a_lane + i * (32 * kRowBytes) + ko[kk]);
-#pragma unroll
-            for (int j = 0; j < NB; ++j) b[j] = *(const frag*)(st + b_lane + j * (32 * kRowBytes) + ko[kk]);
-            // Operands swapped (B rows as the MFMA "A" matrix) so that a lane
-            // ends up with 4 consecutive n for one m: 8-byte stores.
-#pragma unroll
-            for (int i = 0; i < NB; ++i)
-#pragma unroll
-                for (int j = 0; j < NB; ++j) acc[i][j] = Mma<T>::run(b[j], a[i], acc[i][j]);
-        }
-    }
+    frag a0[NB], b0[NB], a1[NB], b1[NB];
 
-    // ---- epilogue: registers -> global -----------------------------------------
+    auto load_frags = [&](int st, int ko, frag(&a)[NB], frag(&b)[NB]) {
+        const unsigned char* base = smem + st * STAGE + ko;
+#pragma unroll
+        for (int i = 0; i < NB; ++i) a[i] = *(const frag*)(base + a_lane + i * BLK);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) b[j] = *(const frag*)(base + b_lane + j * BLK);
+    };
+    // Operands swapped (B rows as the MFMA "A" matrix) so that a lane ends up
+    // with 4 consecutive n for one m.
+    auto mma = [&](frag(&a)[NB], frag(&b)[NB]) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+#pragma unroll
+            for (int j = 0; j < NB; ++j) acc[i][j] = Mma<T>::run(b[j], a[i], acc[i][j]);
+    };
+    // Scheduling hint for one half step of NB*NB MFMAs: the LDS reads of the
+    // next half step go out one per MFMA at the front, so the remaining MFMAs
+    // cover their latency and the wait at the end of the half step does not
+    // stall.  The HBM->LDS copies are placed one per MFMA in slots that differ
+    // from wave to wave (W = wave id): the four waves run in lockstep between
+    // barriers, and copies issued in the same slot queue up behind each other at
+    // the CU's single address unit while the MFMA pipes idle.
+    auto interleave = [&](auto reads_c, auto copies_c, auto wave_c) {
+        constexpr int reads = decltype(reads_c)::value;
+        constexpr int copies = decltype(copies_c)::value;
+        constexpr int W = decltype(wave_c)::value;
+        constexpr int NM = NB * NB;
+#pragma unroll
+        for (int slot = 0; slot < reads && slot < NM; ++slot) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        }
+        if constexpr (NM - reads >= 8 && copies > 0) {
+            // two copy slots per wave in the back half: reads+W and reads+4+W
+#pragma unroll
+            for (int slot = reads; slot < NM; ++slot) {
+                if (slot == reads + W || slot == reads + 4 + W)
+                    __builtin_amdgcn_sched_group_barrier(0x020, copies / 2, 0);  // VMEM reads
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+        } else {
+            if constexpr (copies > 0) __builtin_amdgcn_sched_group_barrier(0x020, copies, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, NM, 0);  // whatever MFMAs are left
+        }
+    };
+    template_int<2 * NB> all_reads;
+    template_int<0> none;
+
+    const int KT = K / kBK;
+    constexpr int AHEAD = NS - 1;   // copies run AHEAD tiles ahead of the MFMAs
+    constexpr int HALF = LPT / 2;   // copies per wave per half tile
+    template_int<0> first_half;
+    template_int<1> second_half;
+    int cur = 0;                    // ring stage of tile kt
+    // One k-step.  The first half step issues the second half of tile kt+AHEAD-1
+    // (COPYA), the second half step the first half of tile kt+AHEAD (COPYB), so
+    // copies are spread evenly between the MFMAs.  NEXT: tile kt+1 exists.  VM:
+    // how many of this wave's copies may still be in flight once tile kt+1 has landed.
+    auto kstep = [&](int kt, auto copya_c, auto copyb_c, auto next_c, auto vm_c, auto wave_c) {
+        constexpr bool COPYA = decltype(copya_c)::value && DBG != 1;
+        constexpr bool COPYB = decltype(copyb_c)::value && DBG != 1;
+        constexpr bool NEXT = decltype(next_c)::value;
+        constexpr int VM = decltype(vm_c)::value;
+        const int nxt = cur + 1 == NS ? 0 : cur + 1;
+        const int prv = cur == 0 ? NS - 1 : cur - 1;   // held tile kt-1, receives tile kt+AHEAD
+        const int prv2 = prv == 0 ? NS - 1 : prv - 1;  // receives tile kt+AHEAD-1
+        if constexpr (DBG != 2) load_frags(cur, ko1, a1, b1);
+        if constexpr (COPYA) issue_half(kt + AHEAD - 1, prv2, second_half);
+        mma(a0, b0);
+        if constexpr (DBG == 2) interleave(none, template_int<(COPYA ? HALF : 0)>{}, wave_c);
+        else interleave(all_reads, template_int<(COPYA ? HALF : 0)>{}, wave_c);
+        __builtin_amdgcn_sched_barrier(0);  // nothing moves across the end of a half step
+        wait_lds_reads();
+        if constexpr (NEXT) {
+            // Tile kt+1 has landed for every wave; every wave is past its reads of
+            // tile kt-1, whose stage the copies of tile kt+AHEAD overwrite.
+            if constexpr (DBG != 4) wait_vmcnt<VM>();
+            if constexpr (DBG != 5) __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (DBG != 2) load_frags(nxt, ko0, a0, b0);
+            if constexpr (COPYB) issue_half(kt + AHEAD, prv, first_half);
+        }
+        mma(a1, b1);
+        if constexpr (NEXT) {
+            if constexpr (DBG == 2) interleave(none, template_int<(COPYB ? HALF : 0)>{}, wave_c);
+            else interleave(all_reads, template_int<(COPYB ? HALF : 0)>{}, wave_c);
+            __builtin_amdgcn_sched_barrier(0);
+            wait_lds_reads();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        cur = nxt;
+    };
+
+    // Prologue: tiles 0 .. AHEAD-2 and the first half of tile AHEAD-1 go out; wait for tile 0.
+    static_for<AHEAD>([&](auto t) {
+        constexpr int tile = decltype(t)::value;
+        if (tile < KT) {
+            issue_half(tile, tile, first_half);
+            if (tile < AHEAD - 1) issue_half(tile, tile, second_half);
+        }
+    });
+    if (KT >= AHEAD) wait_vmcnt<(AHEAD - 2) * LPT + HALF>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    load_frags(0, ko0, a0, b0);
+    wait_lds_reads();
+
+    constexpr int VM_MAIN = (DBG == 1 ? 0 : (AHEAD - 2) * LPT);
+    // The same loop four times over, one copy per wave id, differing only in the
+    // slots the copies are scheduled into.
+    static_for<4>([&](auto wave_c) {
+        if (wave != decltype(wave_c)::value) return;
+        int kt = 0;
+        for (; kt < KT - AHEAD; ++kt)
+            kstep(kt, std::true_type{}, std::true_type{}, std::true_type{}, template_int<VM_MAIN>{}, wave_c);
+        // Tail: r tiles remain after this one, r = min(AHEAD-1, KT-1) .. 0.
+        static_for<AHEAD>([&](auto t) {
+            constexpr int r = AHEAD - 1 - decltype(t)::value;
+            constexpr int ahead = (r - 1 < AHEAD - 2 ? r - 1 : AHEAD - 2);
+            constexpr int vm = (DBG == 1 || ahead < 0) ? 0 : ahead * LPT;
+            if (KT - 1 - kt == r) {
+                // the second half of the last tile is still to be issued when exactly AHEAD-1 remain
+                kstep(kt, std::integral_constant<bool, (r == AHEAD - 1)>{}, std::false_type{},
+                      std::integral_constant<bool, (r > 0)>{}, template_int<vm>{}, wave_c);
+                ++kt;
+            }
+        });
+    });
+
+    // ---- epilogue: registers -> LDS strip -> global -------------------------------
     // acc[i][j][4q+r] is element m = 32i + l%32, n = 32j + 8q + 4(l/32) + r.
+    __syncthreads();  // every wave is done with the stage buffers
+    constexpr int PITCH = WT * 2 + 16;                  // strip row pitch in bytes
+    constexpr int ROWCH = WT / 8;                       // 16-byte chunks per strip row
+    unsigned char* ep = smem + wave * (32 * PITCH);
     T* D = (T*)p.D;
+    [[maybe_unused]] __amdgpu_buffer_rsrc_t drsrc;
+    if constexpr (STORE == 1) drsrc = __builtin_amdgcn_make_buffer_rsrc(p.D, 0, 0xffffffff, 0x00020000);
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-        int row = row0 + 32 * i + fr_row;
-        if constexpr (MODE == kScatter) row = p.RE[row];
-        T* drow = D + (size_t)row * ld + col0 + 4 * fr_h;
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
@@ -220,20 +384,36 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
                 out4 o;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) o[r] = (T)acc[i][j][4 * q + r];
-                *(out4*)(drow + 32 * j + 8 * q) = o;
+                *(out4*)(ep + fr_row * PITCH + (32 * j + 8 * q + 4 * fr_h) * 2) = o;
             }
+#pragma unroll
+        for (int it = 0; it < WT / 16; ++it) {
+            const int c = it * 64 + lane;
+            const int r = c / ROWCH, cc = c % ROWCH;
+            const u32x4 v = *(const u32x4*)(ep + r * PITCH + cc * 16);
+            int row = row0 + 32 * i + r;
+            if constexpr (MODE == kScatter) row = p.RE[row];
+            const size_t off = (size_t)row * ld + col0 + cc * 8;
+            if constexpr (STORE == 1)
+                __builtin_amdgcn_raw_buffer_store_b128(v, drsrc, (int)(off * 2), 0, 16);  // sc1: write-through
+            else
+                *(u32x4*)(D + off) = v;
+        }
     }
 
     // ---- signal ---------------------------------------------------------------------
     if constexpr (MODE != kPlain) {
-        // Every wave's tile stores are acknowledged by L2 before the barrier;
-        // the release on the atomic then writes them back device-wide before
+        // Every wave's tile stores are acknowledged before the barrier; the
+        // release on the atomic then makes them visible device-wide before
         // the counter moves.
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wait_vmcnt<0>();
         __syncthreads();
         const int ntile = (MT / p.BM) * (MT / p.BN);
         if (tid < ntile) {
-            __hip_atomic_fetch_add(p.MM + sig_group, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            if constexpr (REL == 1)  // the stores already went through to memory
+                __hip_atomic_fetch_add(p.MM + sig_group, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else
+                __hip_atomic_fetch_add(p.MM + sig_group, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
             if (p.monitor) {
                 const int order =
                     __hip_atomic_fetch_add(p.MM + p.TN - 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -243,10 +423,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     }
 }
 
-template <typename T, int MT, int MODE>
+template <typename T, int MT, int MODE, int STORE, int REL, int NS, int DBG>
 static int launch_one(const GemmParams& p, hipStream_t stream) {
-    constexpr int smem_bytes = 2 * 2 * MT * kRowBytes;
-    auto kern = gemm_kernel<T, MT, MODE>;
+    constexpr int smem_bytes = NS * 2 * MT * kRowBytes;
+    static_assert(4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the stage buffers");
+    auto kern = gemm_kernel<T, MT, MODE, STORE, REL, NS, DBG>;
     static bool configured = false;  // attribute is per function, set once
     if (!configured) {
         FO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes));
@@ -257,11 +438,36 @@ static int launch_one(const GemmParams& p, hipStream_t stream) {
     return FO_OK;
 }
 
-template <int MODE>
-static int launch_mode(int dtype, int macro, const GemmParams& p, hipStream_t stream) {
-    if (dtype == FO_F16)
-        return macro == 256 ? launch_one<_Float16, 256, MODE>(p, stream) : launch_one<_Float16, 128, MODE>(p, stream);
-    return macro == 256 ? launch_one<__bf16, 256, MODE>(p, stream) : launch_one<__bf16, 128, MODE>(p, stream);
+template <typename T, int MT, int NS>
+static int launch_ns(int mode, const GemmParams& p, hipStream_t stream) {
+    const int store = mode == kPlain ? (g_store_mode ? 1 : 0) : (g_store_mode || g_release_mode ? 1 : 0);
+    const int rel = (mode != kPlain && g_release_mode) ? 1 : 0;
+    if (mode == kPlain)
+        return store ? launch_one<T, MT, kPlain, 1, 0, NS, 0>(p, stream) : launch_one<T, MT, kPlain, 0, 0, NS, 0>(p, stream);
+    if (mode == kSignal) {
+        if (rel) return launch_one<T, MT, kSignal, 1, 1, NS, 0>(p, stream);
+        return store ? launch_one<T, MT, kSignal, 1, 0, NS, 0>(p, stream) : launch_one<T, MT, kSignal, 0, 0, NS, 0>(p, stream);
+    }
+    if (rel) return launch_one<T, MT, kScatter, 1, 1, NS, 0>(p, stream);
+    return store ? launch_one<T, MT, kScatter, 1, 0, NS, 0>(p, stream) : launch_one<T, MT, kScatter, 0, 0, NS, 0>(p, stream);
+}
+
+template <typename T, int MT>
+static int launch_mt(int mode, const GemmParams& p, hipStream_t stream) {
+    if constexpr (MT == 256 && std::is_same<T, __bf16>::value) {
+        if (mode == kPlain && g_debug == 1) return launch_one<T, MT, kPlain, 0, 0, 4, 1>(p, stream);
+        if (mode == kPlain && g_debug == 2) return launch_one<T, MT, kPlain, 0, 0, 4, 2>(p, stream);
+        if (mode == kPlain && g_debug == 3) return launch_one<T, MT, kPlain, 0, 0, 4, 3>(p, stream);
+        if (mode == kPlain && g_debug == 4) return launch_one<T, MT, kPlain, 0, 0, 4, 4>(p, stream);
+        if (mode == kPlain && g_debug == 5) return launch_one<T, MT, kPlain, 0, 0, 4, 5>(p, stream);
+        if (mode == kPlain && g_debug == 6) return launch_one<T, MT, kPlain, 0, 0, 4, 6>(p, stream);
+        if (mode == kPlain && g_debug == 7) return launch_one<T, MT, kPlain, 0, 0, 4, 7>(p, stream);
+    }
+    if constexpr (MT == 256) {
+        if (g_stages == 5) return launch_ns<T, MT, 5>(mode, p, stream);
+        if (g_stages == 3) return launch_ns<T, MT, 3>(mode, p, stream);
+    }
+    return launch_ns<T, MT, 4>(mode, p, stream);
 }
 
 int choose_macro_tile(int BM, int BN, int M, int N) {
@@ -288,6 +494,9 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
     if (M % BM || N % BN) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d not multiples of the %dx%d tile", M, N, BM, BN);
     if (K % kBK) return fail(FO_ERR_SHAPE, "fo_gemm: K=%d not a multiple of %d", K, kBK);
     if ((long long)M * N >= (1LL << 31)) return fail(FO_ERR_LIMIT, "fo_gemm: M*N=%lld needs 64-bit tile offsets", (long long)M * N);
+    if ((long long)M * K >= (1LL << 31) || (long long)N * K >= (1LL << 31))
+        return fail(FO_ERR_LIMIT, "fo_gemm: an operand of %lld elements exceeds the 4 GiB a buffer descriptor addresses",
+                    (long long)(M > N ? M : N) * K);
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)D) & 15) return fail(FO_ERR_ARG, "fo_gemm: operands must be 16-byte aligned");
     const int macro = choose_macro_tile(BM, BN, M, N);
     if (!macro) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d unsupported for tile %dx%d (need multiples of 256, or 128 with the 128x128 tile)", M, N, BM, BN);
@@ -307,11 +516,9 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
         if (rLDN <= 0 || T % rLDN) return fail(FO_ERR_SHAPE, "fo_gemm_signal: rLDN=%d must divide the %d tiles", rLDN, T);
         if (mode == kScatter && !RE) return fail(FO_ERR_ARG, "fo_gemm_scatter: null RE");
     }
-    switch (mode) {
-        case kPlain: return launch_mode<kPlain>(dtype, macro, p, stream);
-        case kSignal: return launch_mode<kSignal>(dtype, macro, p, stream);
-        default: return launch_mode<kScatter>(dtype, macro, p, stream);
-    }
+    if (dtype == FO_F16)
+        return macro == 256 ? launch_mt<_Float16, 256>(mode, p, stream) : launch_mt<_Float16, 128>(mode, p, stream);
+    return macro == 256 ? launch_mt<__bf16, 256>(mode, p, stream) : launch_mt<__bf16, 128>(mode, p, stream);
 }
 
 int raster_hint(int algo, int M, int N, int* hint) {
@@ -329,6 +536,17 @@ int raster_hint(int algo, int M, int N, int* hint) {
         for (int i = 0; i < tiles_m; ++i)
             for (int j = 0; j < tiles_n; ++j) hint[k++] = (c.m * tiles_m + i) * TN + c.n * tiles_n + j;
     }
+    return FO_OK;
+}
+
+int tune(const char* key, int value) {
+    if (!key) return fail(FO_ERR_ARG, "fo_tune: null key");
+    const std::string_view k(key);
+    if (k == "store_mode") g_store_mode = value ? 1 : 0;
+    else if (k == "release_mode") g_release_mode = value ? 1 : 0;
+    else if (k == "stages" && value >= 3 && value <= 5) g_stages = value;
+    else if (k == "debug" && value >= 0 && value <= 7) g_debug = value;
+    else return fail(FO_ERR_ARG, "fo_tune: unknown knob '%s'", key);
     return FO_OK;
 }
 

@@ -27,6 +27,7 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
                 const int* gtable, const void* A, const void* B, void* D, int* MM, const int* RA,
                 const int* RE, int monitor, hipStream_t stream);
 int raster_hint(int algo, int M, int N, int* hint);
+int tune(const char* key, int value);
 
 // fo_sync.hip
 int launch_group_table(const int* cseg, int G, int T, int* table, hipStream_t stream);

@@ -61,7 +61,7 @@ int fo_device_info(int* cu_count, int* clock_khz, int* xcd_count);
 /* D[M,N] = A[M,K] . B[N,K]^T, fp32 accumulate, natural row-major D.
  * Replaces gemm_func_table[Algo] / mutlass_gemm<TM,TN,TK>
  * (src/tiling/gemm_dispatcher.h:16-20, src/gemm/gemm.cu:29-113).
- * Requires M % BM == 0, N % BN == 0, K % 64 == 0, 16-byte aligned pointers. */
+ * Requires M % BM == 0, N % BN == 0, K % 32 == 0, 16-byte aligned pointers. */
 int fo_gemm(int dtype, int algo, int M, int N, int K,
             const void* A, const void* B, void* D, void* stream);
 
@@ -103,6 +103,14 @@ int fo_build_group_table(const int* cseg_dev, int G, int T, int* group_table, vo
  * the sampled completion order of the reference tuner
  * (tune/search.py:164-263), which exists because its scheduler is opaque. */
 int fo_raster_hint(int algo, int M, int N, int* hint_host);
+
+/* Process-wide tuning knobs of the GEMM epilogue, for measurement; no
+ * counterpart in the reference.  Results are identical for every setting.
+ *   "store_mode"   0: cached tile stores (default); 1: agent-scope
+ *                  write-through tile stores.
+ *   "release_mode" 0: release-ordered signal atomic (default); 1: write-through
+ *                  tile stores, wait for their acknowledgement, relaxed atomic. */
+int fo_tune(const char* key, int value);
 
 /* ---- counting / wait -------------------------------------------------- */
 

@@ -147,8 +147,8 @@ def test_gemm_random_within_tolerance(L, dev, dt):
 
 
 def test_gemm_rejects_unsupported_shapes(L, dev):
-    a = torch.zeros(256, 96, dtype=torch.float16, device=dev)
-    assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 96, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
+    a = torch.zeros(384, 384, dtype=torch.float16, device=dev)  # large enough for every call below
+    assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 48, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
     assert L.fo_gemm(capi.FO_F16, 3, 384, 384, 64, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
 
 
