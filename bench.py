@@ -56,7 +56,7 @@ def main() -> int:
     ap.add_argument("--group-tiles", type=int, default=0, help="tiles per signal group (0 = workload default)")
     ap.add_argument("--kernel-iters", type=int, default=100, help="timed launches per isolated kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline work; 0 skips it")
-    ap.add_argument("--consumer-blocks", type=int, default=8)
+    ap.add_argument("--consumer-blocks", type=int, default=64)
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build drives one GPU only; run with --gpus 1 "

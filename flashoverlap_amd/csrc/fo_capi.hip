@@ -21,7 +21,7 @@ int fail(int code, const char* fmt, ...) {
 
 // Layout tile selected by each Algo index, in the order of the reference's
 // instance list (src/inc/signal_instances.inc:1-6).  The third number is the
-// reference's k-tile; this library always stages 32 k-elements per LDS stage,
+// reference's k-tile; this library always stages 64 k-elements per LDS buffer,
 // so entries that differ only in it select the same kernel.
 static const int kAlgo[][3] = {
     {128, 128, 32}, {128, 128, 64}, {128, 256, 32}, {128, 256, 64}, {256, 128, 32}, {256, 128, 64},

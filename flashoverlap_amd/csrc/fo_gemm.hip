@@ -5,14 +5,18 @@
 // 128 for small problems); each wavefront owns an (MT/2) x (MT/2) quadrant as
 // (MT/64)^2 blocks of v_mfma_f32_32x32x16, accumulators in AGPRs.
 //
-// Main loop: A and B panels of 32 k-elements stream HBM -> LDS with
-// global_load_lds_dwordx4 (no register staging) through a ring of 4 LDS
-// stages, so copies are issued three k-steps ahead of their use.  The 16-byte
-// chunks of a tile row are XOR-swizzled by row so the ds_read_b128 fragment
-// reads are bank-conflict free.  Fragments are double-buffered in registers:
-// while the 16 MFMAs of one half k-step run, the fragments of the next half
-// step (possibly of the next stage) are already being read, and there is one
-// workgroup barrier per k-step.
+// Main loop: A and B panels of 64 k-elements stream HBM -> LDS with
+// buffer_load_dwordx4 ... lds (no register staging) into two LDS buffers.  A
+// panel row is 128 bytes, so every copy instruction fetches eight whole cache
+// lines: the L2 serves one request per channel per clock whatever its size, and
+// at this tile size the kernel sits at the edge of that request rate, so
+// half-line requests cost a quarter of the throughput.  The 16-byte chunks of a
+// row are XOR-swizzled by row so the ds_read_b128 fragment reads are
+// bank-conflict free.  A k-step of 64 is four quarter steps of 16 MFMAs each;
+// fragments are double-buffered in registers, so while one quarter's MFMAs
+// run the next quarter's fragments (in the last quarter: the next panel's) are
+// already being read.  The copies of panel p+2 start as soon as panel p has
+// been read for the last time, and there is one workgroup barrier per k-step.
 //
 // Epilogue: the quadrant goes through LDS in strips of 32 rows so that every
 // global store instruction writes four whole 256-byte row segments, either to
@@ -62,16 +66,14 @@ struct Mma<__bf16> {
     }
 };
 
-constexpr int kBK = 32;             // k-elements per LDS stage
-constexpr int kRowBytes = kBK * 2;  // one tile row in LDS: 64 bytes = 4 chunks of 16
+constexpr int kBK = 64;             // k-elements per LDS buffer
+constexpr int kRowBytes = kBK * 2;  // one panel row in LDS: 128 bytes = 8 chunks of 16
 
 enum { kPlain = 0, kSignal = 1, kScatter = 2 };
 
 // Tuning knobs (fo_tune): how the epilogue stores C and how it signals.
 int g_store_mode = 0;    // 0 = cached stores, 1 = agent-scope write-through stores (sc1)
 int g_release_mode = 0;  // 0 = release-ordered atomic, 1 = write-through stores + relaxed atomic (needs store mode 1)
-int g_stages = 4;        // LDS ring stages of the 256 macro tile (3, 4 or 5)
-int g_debug = 0;         // what-if timing variants of the bf16 256 plain kernel (wrong results)
 
 struct GemmParams {
     const void* A;
@@ -116,8 +118,9 @@ __device__ __forceinline__ int scan_group(const int* cseg, int slot) {
 }
 
 // Row swizzle shared by the copy and the fragment reads: LDS chunk (row, cc)
-// holds k-chunk cc ^ swz(row).  Conflict free for 8 or 16 consecutive rows.
-__device__ __forceinline__ int swz(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+// holds k-chunk cc ^ swz(row).  Any 8 (or, two rows per 256 bytes, any 16)
+// consecutive rows then hit distinct banks when they read the same k-chunk.
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 template <int N>
 using template_int = std::integral_constant<int, N>;
@@ -131,19 +134,16 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
-// STORE: 0 cached, 1 write-through tile stores; REL: 0 release atomic, 1 relaxed atomic;
-// NS: LDS ring stages; DBG: what-if timing variants that compute wrong results
-// (1 = no HBM->LDS copies in the main loop, 2 = no LDS fragment reads in the main loop,
-// 3 = every copy re-reads tile 0, 4 = no wait for the copies, 5 = no barrier in the main loop,
-// 6 = every copy re-reads the same 2 KiB, 7 = copies fetch whole 128-byte lines).
-template <typename T, int MT, int MODE, int STORE, int REL, int NS, int DBG>
+// STORE: 0 cached, 1 write-through tile stores; REL: 0 release atomic, 1 relaxed atomic.
+template <typename T, int MT, int MODE, int STORE, int REL>
 __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     constexpr int WT = MT / 2;               // wave quadrant edge
     constexpr int NB = WT / 32;              // 32x32 MFMA blocks per quadrant edge
-    constexpr int PANEL = MT * kRowBytes;    // bytes of one A (or B) panel per stage
-    constexpr int STAGE = 2 * PANEL;
-    constexpr int LOADS = MT / 64;           // wave-wide 1 KiB copies per wave per panel
+    constexpr int PANEL = MT * kRowBytes;    // bytes of one A (or B) panel
+    constexpr int BUF = 2 * PANEL;           // one LDS buffer: A panel, then B panel
+    constexpr int LOADS = MT / 32;           // wave-wide 1 KiB copies per wave per panel
     constexpr int LPT = 2 * LOADS;           // copies per wave per k-step
+    constexpr int HALF = LPT / 2;
     constexpr int BLK = 32 * kRowBytes;      // LDS bytes between 32-row blocks
     using frag = typename Mma<T>::frag;
     using out4 = typename Mma<T>::out4;
@@ -186,36 +186,38 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         }
     }
 
-    // ---- global -> LDS copy addressing ---------------------------------------
-    // A wave-wide copy fills 64 consecutive 16-byte LDS chunks = 16 tile rows.
-    const int cp_row = lane >> 2;                      // row within the 16-row slab
-    const int cp_kc = (lane & 3) ^ swz(cp_row);        // k-chunk this lane fetches
-    // Buffer addressing: the operand is the buffer, the wave-uniform part of the
-    // offset (tile row, slab, k) lives in a scalar register and only the constant
-    // per-lane part in a vector register, so a copy costs no vector ALU work.
-    const int cp_off = DBG == 7 ? ((lane >> 3) * K + (lane & 7) * 8) * 2   // what-if: 8 rows x 128 B per copy
-                                : (cp_row * K + cp_kc * 8) * 2;
+    // ---- HBM -> LDS copy addressing ------------------------------------------
+    // One copy instruction moves 1 KiB = 8 panel rows of 128 bytes: lane l's 16
+    // bytes land at the LDS base + 16*l, i.e. row l/8, chunk l%8 of the slab, and
+    // are fetched from k-chunk (l%8) ^ swz(row).  Buffer addressing: the operand
+    // is the buffer, the wave-uniform part of the offset (panel row, slab, k)
+    // lives in a scalar register and only the constant per-lane part in a vector
+    // register, so a copy costs no vector ALU work.  Slabs alternate in bit 3 of
+    // the row number, hence two per-lane offsets.
+    const int cp_row = lane >> 3;
+    const int cp_off0 = (cp_row * K + ((lane & 7) ^ swz(cp_row)) * 8) * 2;       // even slabs
+    const int cp_off1 = (cp_row * K + ((lane & 7) ^ swz(cp_row + 8)) * 8) * 2;   // odd slabs
     const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, 0xffffffff, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, 0xffffffff, 0x00020000);
-    const unsigned baseA = (unsigned)(mt.m * MT + wave * (LOADS * 16)) * (unsigned)K * 2u;
-    const unsigned baseB = (unsigned)(mt.n * MT + wave * (LOADS * 16)) * (unsigned)K * 2u;
-    const unsigned slab_bytes = 16u * (unsigned)K * 2u;   // bytes between consecutive slabs
+    const unsigned baseA = (unsigned)(mt.m * MT + wave * (LOADS * 8)) * (unsigned)K * 2u;
+    const unsigned baseB = (unsigned)(mt.n * MT + wave * (LOADS * 8)) * (unsigned)K * 2u;
+    const unsigned slab_bytes = 8u * (unsigned)K * 2u;    // bytes between consecutive slabs
     const int lds_cp = wave * (LOADS * 1024);             // this wave's first slab in a panel
 
-    // Stage `st` of the ring receives tile `kt`; the copies of a tile are issued
-    // in two halves so that they can be spread over a whole k-step.  One copy
-    // moves 1 KiB: lane l's 16 bytes land at the LDS address + 16*l.
-    auto issue_half = [&](int kt, int st, auto half_c) {
+    // Buffer `buf` receives panel `kt`; the copies of a panel are issued in two
+    // halves so that they can be spread over two quarter steps.
+    auto issue_half = [&](int kt, int buf, auto half_c) {
         constexpr int H = decltype(half_c)::value;
-        unsigned char* sA = smem + st * STAGE + lds_cp;
+        unsigned char* sA = smem + buf * BUF + lds_cp;
         unsigned char* sB = sA + PANEL;
-        const unsigned koff = (unsigned)(DBG == 3 ? 0 : kt) * (DBG == 7 ? 128 : kBK * 2) % (unsigned)(K * 2);
+        const unsigned koff = (unsigned)kt * (kBK * 2);
 #pragma unroll
         for (int j = H * (LOADS / 2); j < (H + 1) * (LOADS / 2); ++j) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(sA + j * 1024), 16, cp_off,
-                                                     (int)(baseA + (DBG == 6 ? 0 : j * slab_bytes + koff)), 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(sB + j * 1024), 16, cp_off,
-                                                     (int)(baseB + (DBG == 6 ? 0 : j * slab_bytes + koff)), 0, 0);
+            const int voff = (j & 1) ? cp_off1 : cp_off0;   // LOADS*8 is a multiple of 16: slab parity = j parity
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(sA + j * 1024), 16, voff,
+                                                     (int)(baseA + j * slab_bytes + koff), 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(sB + j * 1024), 16, voff,
+                                                     (int)(baseB + j * slab_bytes + koff), 0, 0);
         }
     };
 
@@ -224,8 +226,9 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     const int fr_row = lane & 31, fr_h = lane >> 5;
     const int a_lane = (wm * WT + fr_row) * kRowBytes;
     const int b_lane = PANEL + (wn * WT + fr_row) * kRowBytes;
-    const int ko0 = ((0 + fr_h) ^ swz(fr_row)) * 16;   // first half k-step (k 0..15)
-    const int ko1 = ((2 + fr_h) ^ swz(fr_row)) * 16;   // second half (k 16..31)
+    int ko[4];   // chunk offset of each quarter step (k 0..15, 16..31, 32..47, 48..63)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) ko[q] = ((2 * q + fr_h) ^ swz(fr_row)) * 16;
 
     f32x16 acc[NB][NB];
 #pragma unroll
@@ -237,8 +240,8 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 
     frag a0[NB], b0[NB], a1[NB], b1[NB];
 
-    auto load_frags = [&](int st, int ko, frag(&a)[NB], frag(&b)[NB]) {
-        const unsigned char* base = smem + st * STAGE + ko;
+    auto load_frags = [&](int buf, int kofs, frag(&a)[NB], frag(&b)[NB]) {
+        const unsigned char* base = smem + buf * BUF + kofs;
 #pragma unroll
         for (int i = 0; i < NB; ++i) a[i] = *(const frag*)(base + a_lane + i * BLK);
 #pragma unroll
@@ -252,123 +255,102 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int j = 0; j < NB; ++j) acc[i][j] = Mma<T>::run(b[j], a[i], acc[i][j]);
     };
-    // Scheduling hint for one half step of NB*NB MFMAs: the LDS reads of the
-    // next half step go out one per MFMA at the front, so the remaining MFMAs
-    // cover their latency and the wait at the end of the half step does not
-    // stall.  The HBM->LDS copies are placed one per MFMA in slots that differ
-    // from wave to wave (W = wave id): the four waves run in lockstep between
-    // barriers, and copies issued in the same slot queue up behind each other at
-    // the CU's single address unit while the MFMA pipes idle.
-    auto interleave = [&](auto reads_c, auto copies_c, auto wave_c) {
+    // Scheduling hint for one quarter step of NB*NB MFMAs: the LDS reads of the
+    // next quarter go out one per MFMA at the front, so the remaining MFMAs
+    // cover their latency and the wait at the end of the quarter does not stall;
+    // the HBM->LDS copies follow, one per MFMA.
+    auto interleave = [&](auto reads_c, auto copies_c) {
         constexpr int reads = decltype(reads_c)::value;
         constexpr int copies = decltype(copies_c)::value;
-        constexpr int W = decltype(wave_c)::value;
         constexpr int NM = NB * NB;
 #pragma unroll
         for (int slot = 0; slot < reads && slot < NM; ++slot) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one DS read
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
         }
-        if constexpr (NM - reads >= 8 && copies > 0) {
-            // two copy slots per wave in the back half: reads+W and reads+4+W
+        if constexpr (copies > 0 && reads < NM) {
+            constexpr int per_slot = (copies + (NM - reads) - 1) / (NM - reads);
 #pragma unroll
-            for (int slot = reads; slot < NM; ++slot) {
-                if (slot == reads + W || slot == reads + 4 + W)
-                    __builtin_amdgcn_sched_group_barrier(0x020, copies / 2, 0);  // VMEM reads
+            for (int i = 0; i < copies; i += per_slot) {
+                __builtin_amdgcn_sched_group_barrier(0x020, per_slot, 0);  // VMEM reads
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             }
-        } else {
-            if constexpr (copies > 0) __builtin_amdgcn_sched_group_barrier(0x020, copies, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, NM, 0);  // whatever MFMAs are left
+        } else if constexpr (copies > 0) {
+            __builtin_amdgcn_sched_group_barrier(0x020, copies, 0);
         }
+        __builtin_amdgcn_sched_group_barrier(0x008, NM, 0);  // whatever MFMAs are left
     };
     template_int<2 * NB> all_reads;
     template_int<0> none;
-
-    const int KT = K / kBK;
-    constexpr int AHEAD = NS - 1;   // copies run AHEAD tiles ahead of the MFMAs
-    constexpr int HALF = LPT / 2;   // copies per wave per half tile
     template_int<0> first_half;
     template_int<1> second_half;
-    int cur = 0;                    // ring stage of tile kt
-    // One k-step.  The first half step issues the second half of tile kt+AHEAD-1
-    // (COPYA), the second half step the first half of tile kt+AHEAD (COPYB), so
-    // copies are spread evenly between the MFMAs.  NEXT: tile kt+1 exists.  VM:
-    // how many of this wave's copies may still be in flight once tile kt+1 has landed.
-    auto kstep = [&](int kt, auto copya_c, auto copyb_c, auto next_c, auto vm_c, auto wave_c) {
-        constexpr bool COPYA = decltype(copya_c)::value && DBG != 1;
-        constexpr bool COPYB = decltype(copyb_c)::value && DBG != 1;
-        constexpr bool NEXT = decltype(next_c)::value;
-        constexpr int VM = decltype(vm_c)::value;
-        const int nxt = cur + 1 == NS ? 0 : cur + 1;
-        const int prv = cur == 0 ? NS - 1 : cur - 1;   // held tile kt-1, receives tile kt+AHEAD
-        const int prv2 = prv == 0 ? NS - 1 : prv - 1;  // receives tile kt+AHEAD-1
-        if constexpr (DBG != 2) load_frags(cur, ko1, a1, b1);
-        if constexpr (COPYA) issue_half(kt + AHEAD - 1, prv2, second_half);
-        mma(a0, b0);
-        if constexpr (DBG == 2) interleave(none, template_int<(COPYA ? HALF : 0)>{}, wave_c);
-        else interleave(all_reads, template_int<(COPYA ? HALF : 0)>{}, wave_c);
-        __builtin_amdgcn_sched_barrier(0);  // nothing moves across the end of a half step
+
+    // One quarter step: read the fragments of the next quarter into (an, bn),
+    // optionally issue half a panel of copies, run the MFMAs on (ac, bc).
+    auto quarter = [&](int rbuf, int rko, frag(&an)[NB], frag(&bn)[NB], frag(&ac)[NB], frag(&bc)[NB], auto read_c,
+                       auto copy_c, int ckt, int cbuf, auto half_c) {
+        constexpr bool READ = decltype(read_c)::value;
+        constexpr bool COPY = decltype(copy_c)::value;
+        if constexpr (READ) load_frags(rbuf, rko, an, bn);
+        if constexpr (COPY) issue_half(ckt, cbuf, half_c);
+        mma(ac, bc);
+        constexpr int ncopy = COPY ? HALF : 0;
+        if constexpr (READ) interleave(all_reads, template_int<ncopy>{});
+        else interleave(none, template_int<ncopy>{});
+        __builtin_amdgcn_sched_barrier(0);  // nothing moves across the end of a quarter step
         wait_lds_reads();
-        if constexpr (NEXT) {
-            // Tile kt+1 has landed for every wave; every wave is past its reads of
-            // tile kt-1, whose stage the copies of tile kt+AHEAD overwrite.
-            if constexpr (DBG != 4) wait_vmcnt<VM>();
-            if constexpr (DBG != 5) __builtin_amdgcn_s_barrier();
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (DBG != 2) load_frags(nxt, ko0, a0, b0);
-            if constexpr (COPYB) issue_half(kt + AHEAD, prv, first_half);
-        }
-        mma(a1, b1);
-        if constexpr (NEXT) {
-            if constexpr (DBG == 2) interleave(none, template_int<(COPYB ? HALF : 0)>{}, wave_c);
-            else interleave(all_reads, template_int<(COPYB ? HALF : 0)>{}, wave_c);
-            __builtin_amdgcn_sched_barrier(0);
-            wait_lds_reads();
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        cur = nxt;
+        __builtin_amdgcn_sched_barrier(0);
     };
 
-    // Prologue: tiles 0 .. AHEAD-2 and the first half of tile AHEAD-1 go out; wait for tile 0.
-    static_for<AHEAD>([&](auto t) {
-        constexpr int tile = decltype(t)::value;
-        if (tile < KT) {
-            issue_half(tile, tile, first_half);
-            if (tile < AHEAD - 1) issue_half(tile, tile, second_half);
+    const int NP = K / kBK;   // panels
+    // One k-step on panel kt (in buffer cur).  C1: panel kt+1 exists and its second
+    // half is still to be copied.  NEXT: panel kt+1 exists.  C2: panel kt+2 exists.
+    auto kstep = [&](int kt, int cur, auto c1_c, auto next_c, auto c2_c) {
+        constexpr bool NEXT = decltype(next_c)::value;
+        quarter(cur, ko[1], a1, b1, a0, b0, std::true_type{}, c1_c, kt + 1, cur ^ 1, second_half);
+        quarter(cur, ko[2], a0, b0, a1, b1, std::true_type{}, std::false_type{}, 0, 0, first_half);
+        quarter(cur, ko[3], a1, b1, a0, b0, std::true_type{}, std::false_type{}, 0, 0, first_half);
+        if constexpr (NEXT) {
+            // Panel kt+1 has landed for every wave, and every wave has read panel kt
+            // for the last time, so its buffer can take panel kt+2.
+            wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            quarter(cur ^ 1, ko[0], a0, b0, a1, b1, std::true_type{}, c2_c, kt + 2, cur, first_half);
+        } else {
+            quarter(0, 0, a0, b0, a1, b1, std::false_type{}, std::false_type{}, 0, 0, first_half);
         }
-    });
-    if (KT >= AHEAD) wait_vmcnt<(AHEAD - 2) * LPT + HALF>();
-    else wait_vmcnt<0>();
+    };
+
+    // Prologue: panel 0 and the first half of panel 1 go out; wait for panel 0.
+    issue_half(0, 0, first_half);
+    issue_half(0, 0, second_half);
+    if (NP > 1) {
+        issue_half(1, 1, first_half);
+        wait_vmcnt<HALF>();
+    } else {
+        wait_vmcnt<0>();
+    }
     __builtin_amdgcn_s_barrier();
-    load_frags(0, ko0, a0, b0);
+    load_frags(0, ko[0], a0, b0);
     wait_lds_reads();
 
-    constexpr int VM_MAIN = (DBG == 1 ? 0 : (AHEAD - 2) * LPT);
-    // The same loop four times over, one copy per wave id, differing only in the
-    // slots the copies are scheduled into.
-    static_for<4>([&](auto wave_c) {
-        if (wave != decltype(wave_c)::value) return;
-        int kt = 0;
-        for (; kt < KT - AHEAD; ++kt)
-            kstep(kt, std::true_type{}, std::true_type{}, std::true_type{}, template_int<VM_MAIN>{}, wave_c);
-        // Tail: r tiles remain after this one, r = min(AHEAD-1, KT-1) .. 0.
-        static_for<AHEAD>([&](auto t) {
-            constexpr int r = AHEAD - 1 - decltype(t)::value;
-            constexpr int ahead = (r - 1 < AHEAD - 2 ? r - 1 : AHEAD - 2);
-            constexpr int vm = (DBG == 1 || ahead < 0) ? 0 : ahead * LPT;
-            if (KT - 1 - kt == r) {
-                // the second half of the last tile is still to be issued when exactly AHEAD-1 remain
-                kstep(kt, std::integral_constant<bool, (r == AHEAD - 1)>{}, std::false_type{},
-                      std::integral_constant<bool, (r > 0)>{}, template_int<vm>{}, wave_c);
-                ++kt;
-            }
-        });
-    });
+    // The consumer's waves share SIMDs with these waves while a group is being
+    // copied; the issue arbiter should always prefer the wave that feeds the MFMAs.
+    __builtin_amdgcn_s_setprio(3);
+    int kt = 0, cur = 0;
+    for (; kt < NP - 2; ++kt, cur ^= 1) kstep(kt, cur, std::true_type{}, std::true_type{}, std::true_type{});
+    if (NP >= 2) {
+        kstep(kt, cur, std::true_type{}, std::true_type{}, std::false_type{});
+        ++kt;
+        cur ^= 1;
+    }
+    kstep(kt, cur, std::false_type{}, std::false_type{}, std::false_type{});
 
     // ---- epilogue: registers -> LDS strip -> global -------------------------------
     // acc[i][j][4q+r] is element m = 32i + l%32, n = 32j + 8q + 4(l/32) + r.
-    __syncthreads();  // every wave is done with the stage buffers
+    __builtin_amdgcn_s_setprio(0);
+    __syncthreads();  // every wave is done with the panel buffers
     constexpr int PITCH = WT * 2 + 16;                  // strip row pitch in bytes
     constexpr int ROWCH = WT / 8;                       // 16-byte chunks per strip row
     unsigned char* ep = smem + wave * (32 * PITCH);
@@ -423,11 +405,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     }
 }
 
-template <typename T, int MT, int MODE, int STORE, int REL, int NS, int DBG>
+template <typename T, int MT, int MODE, int STORE, int REL>
 static int launch_one(const GemmParams& p, hipStream_t stream) {
-    constexpr int smem_bytes = NS * 2 * MT * kRowBytes;
-    static_assert(4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the stage buffers");
-    auto kern = gemm_kernel<T, MT, MODE, STORE, REL, NS, DBG>;
+    constexpr int smem_bytes = 2 * 2 * MT * kRowBytes;
+    static_assert(4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the panel buffers");
+    auto kern = gemm_kernel<T, MT, MODE, STORE, REL>;
     static bool configured = false;  // attribute is per function, set once
     if (!configured) {
         FO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes));
@@ -438,36 +420,18 @@ static int launch_one(const GemmParams& p, hipStream_t stream) {
     return FO_OK;
 }
 
-template <typename T, int MT, int NS>
-static int launch_ns(int mode, const GemmParams& p, hipStream_t stream) {
+template <typename T, int MT>
+static int launch_mt(int mode, const GemmParams& p, hipStream_t stream) {
     const int store = mode == kPlain ? (g_store_mode ? 1 : 0) : (g_store_mode || g_release_mode ? 1 : 0);
     const int rel = (mode != kPlain && g_release_mode) ? 1 : 0;
     if (mode == kPlain)
-        return store ? launch_one<T, MT, kPlain, 1, 0, NS, 0>(p, stream) : launch_one<T, MT, kPlain, 0, 0, NS, 0>(p, stream);
+        return store ? launch_one<T, MT, kPlain, 1, 0>(p, stream) : launch_one<T, MT, kPlain, 0, 0>(p, stream);
     if (mode == kSignal) {
-        if (rel) return launch_one<T, MT, kSignal, 1, 1, NS, 0>(p, stream);
-        return store ? launch_one<T, MT, kSignal, 1, 0, NS, 0>(p, stream) : launch_one<T, MT, kSignal, 0, 0, NS, 0>(p, stream);
+        if (rel) return launch_one<T, MT, kSignal, 1, 1>(p, stream);
+        return store ? launch_one<T, MT, kSignal, 1, 0>(p, stream) : launch_one<T, MT, kSignal, 0, 0>(p, stream);
     }
-    if (rel) return launch_one<T, MT, kScatter, 1, 1, NS, 0>(p, stream);
-    return store ? launch_one<T, MT, kScatter, 1, 0, NS, 0>(p, stream) : launch_one<T, MT, kScatter, 0, 0, NS, 0>(p, stream);
-}
-
-template <typename T, int MT>
-static int launch_mt(int mode, const GemmParams& p, hipStream_t stream) {
-    if constexpr (MT == 256 && std::is_same<T, __bf16>::value) {
-        if (mode == kPlain && g_debug == 1) return launch_one<T, MT, kPlain, 0, 0, 4, 1>(p, stream);
-        if (mode == kPlain && g_debug == 2) return launch_one<T, MT, kPlain, 0, 0, 4, 2>(p, stream);
-        if (mode == kPlain && g_debug == 3) return launch_one<T, MT, kPlain, 0, 0, 4, 3>(p, stream);
-        if (mode == kPlain && g_debug == 4) return launch_one<T, MT, kPlain, 0, 0, 4, 4>(p, stream);
-        if (mode == kPlain && g_debug == 5) return launch_one<T, MT, kPlain, 0, 0, 4, 5>(p, stream);
-        if (mode == kPlain && g_debug == 6) return launch_one<T, MT, kPlain, 0, 0, 4, 6>(p, stream);
-        if (mode == kPlain && g_debug == 7) return launch_one<T, MT, kPlain, 0, 0, 4, 7>(p, stream);
-    }
-    if constexpr (MT == 256) {
-        if (g_stages == 5) return launch_ns<T, MT, 5>(mode, p, stream);
-        if (g_stages == 3) return launch_ns<T, MT, 3>(mode, p, stream);
-    }
-    return launch_ns<T, MT, 4>(mode, p, stream);
+    if (rel) return launch_one<T, MT, kScatter, 1, 1>(p, stream);
+    return store ? launch_one<T, MT, kScatter, 1, 0>(p, stream) : launch_one<T, MT, kScatter, 0, 0>(p, stream);
 }
 
 int choose_macro_tile(int BM, int BN, int M, int N) {
@@ -544,8 +508,6 @@ int tune(const char* key, int value) {
     const std::string_view k(key);
     if (k == "store_mode") g_store_mode = value ? 1 : 0;
     else if (k == "release_mode") g_release_mode = value ? 1 : 0;
-    else if (k == "stages" && value >= 3 && value <= 5) g_stages = value;
-    else if (k == "debug" && value >= 0 && value <= 7) g_debug = value;
     else return fail(FO_ERR_ARG, "fo_tune: unknown knob '%s'", key);
     return FO_OK;
 }

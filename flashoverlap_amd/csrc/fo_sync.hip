@@ -3,12 +3,16 @@
 //
 // The GEMM epilogue bumps MM[g] with a release-ordered agent-scope atomic once
 // a tile of group g is visible device-wide.  The kernels here run on a second
-// stream while the GEMM is still executing: they poll MM[g] with acquire loads
-// (MI355X has one L2 per XCD and they are not coherent with each other, so the
-// acquire's cache invalidate is what makes the tile data readable), release
-// the group to the consumer once the count is reached, and put the counter
-// back to zero for the next call.  Every wait is bounded in wall-clock time so
-// that a wrong cSeg can delay a stream but never hang the device.
+// stream while the GEMM is still executing.  MI355X has one L2 per XCD and they
+// are not coherent with each other, so a reader on another XCD must not hit a
+// stale line.  An acquire would do that by invalidating its caches - including
+// the A/B panels that the GEMM workgroups of that XCD are sharing through the
+// same L2, once per poll.  So the counters are polled with relaxed agent-scope
+// loads (which bypass the non-coherent caches and invalidate nothing), and the
+// persistent consumer then reads the released tiles with agent-scope coherent
+// loads as well; nothing is invalidated while the GEMM runs.  Every wait is
+// bounded in wall-clock time so that a wrong cSeg can delay a stream but never
+// hang the device.
 #include <hip/hip_runtime.h>
 
 #include "fo_internal.h"
@@ -24,7 +28,7 @@ template <typename Pred>
 __device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, Pred pred) {
     const long long t0 = wall_clock64();
     for (;;) {
-        const int v = __hip_atomic_load(addr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        const int v = __hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (pred(v)) return true;
         if (wall_clock64() - t0 > ticks) return false;
         __builtin_amdgcn_s_sleep(8);
@@ -34,7 +38,8 @@ __device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, P
 // Counterpart of the reference's kernel_wait_flag (src/wait.cuh:5-9): returns
 // once *addr == that and leaves 0 there.  Nothing else writes *addr between
 // the last tile's signal and the reset, so load-then-store equals the
-// reference's compare-and-swap.
+// reference's compare-and-swap.  The kernel that follows on the stream sees
+// the group's tiles through the cache invalidation at its own start.
 __global__ void wait_kernel(int that, int* addr, long long ticks) {
     if (threadIdx.x != 0) return;
     if (bounded_poll(addr, ticks, [that](int v) { return v == that; }))
@@ -43,19 +48,54 @@ __global__ void wait_kernel(int that, int* addr, long long ticks) {
         atomicAdd(&g_wait_timeouts, 1);
 }
 
+constexpr int kCopyThreads = 512;  // consumer workgroup size
+constexpr int kCopyUnroll = 8;     // 16-byte units in flight per thread
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Copies n 16-byte units (n * 16 < 4 GiB); the workgroups of the grid interleave
+// in chunks of kCopyThreads * kCopyUnroll units, every thread keeping kCopyUnroll
+// loads in flight.  COHERENT: read with agent-scope loads that do not hit in
+// the non-coherent caches (for data another XCD wrote while this kernel runs).
+template <bool COHERENT>
+__device__ __forceinline__ void grid_copy(const uint4* __restrict__ s, uint4* __restrict__ d, long long n) {
+    const long long chunk = (long long)kCopyThreads * kCopyUnroll;
+    [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc;
+    if constexpr (COHERENT) rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, 0xffffffff, 0x00020000);
+    for (long long base = (long long)blockIdx.x * chunk; base < n; base += (long long)gridDim.x * chunk) {
+        u32x4 v[kCopyUnroll];
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) {
+            const long long i = base + u * kCopyThreads + threadIdx.x;
+            if (i < n) {
+                if constexpr (COHERENT) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(i * 16), 0, 16);  // sc1
+                else v[u] = *(const u32x4*)(s + i);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kCopyUnroll; ++u) {
+            const long long i = base + u * kCopyThreads + threadIdx.x;
+            if (i < n) *(u32x4*)(d + i) = v[u];
+        }
+    }
+}
+
 // Persistent form of the host loop in src/overlap_impl.cu:257-265 (and
 // :312-323 for the ReduceScatter receive layout): walks the groups in index
 // order; all workgroups cooperate on each group's copy.  A group's range is
 // cut into nslices equal parts; parts slice_first .. slice_first+slice_count-1
 // are copied, part k to dst + (k - slice_first)*stride + offset/nslices (the
-// receive layout of a ReduceScatter; nslices = 1 is the plain copy).  After its stripe a
-// workgroup bumps MM[g] once more; the workgroup that brings it to
-// cSeg[g] + gridDim.x is the last one out and stores the 0.
-__global__ void __launch_bounds__(256) wait_consume_kernel(const int* __restrict__ cseg, int G, int* MM,
-                                                           const uint4* __restrict__ src, uint4* __restrict__ dst,
-                                                           long long tile_units, int nslices, int slice_first,
-                                                           int slice_count, long long slice_stride_units,
-                                                           int* order_log, long long ticks) {
+// receive layout of a ReduceScatter; nslices = 1 is the plain copy).  After its
+// stripe a workgroup bumps MM[g] once more; the workgroup that brings it to
+// cSeg[g] + gridDim.x is the last one out and stores the 0.  It needs few
+// registers and no LDS to speak of, so its waves fit beside a resident GEMM
+// workgroup on the same CU.
+__global__ void __launch_bounds__(kCopyThreads) wait_consume_kernel(const int* __restrict__ cseg, int G, int* MM,
+                                                                    const uint4* __restrict__ src,
+                                                                    uint4* __restrict__ dst, long long tile_units,
+                                                                    int nslices, int slice_first, int slice_count,
+                                                                    long long slice_stride_units, int* order_log,
+                                                                    long long ticks) {
     __shared__ int s_ok;
     const int tid = threadIdx.x;
     long long lo = 0;  // first 16-byte unit of group g in src
@@ -70,12 +110,8 @@ __global__ void __launch_bounds__(256) wait_consume_kernel(const int* __restrict
         if (!s_ok) return;  // uniform: the whole workgroup leaves
         const long long units = tile_units * need;
         const long long part = units / nslices;
-        for (int k = 0; k < slice_count; ++k) {
-            const uint4* s = src + lo + (slice_first + k) * part;
-            uint4* d = dst + k * slice_stride_units + lo / nslices;
-            for (long long i = (long long)blockIdx.x * 256 + tid; i < part; i += (long long)gridDim.x * 256)
-                d[i] = s[i];
-        }
+        for (int k = 0; k < slice_count; ++k)
+            grid_copy<true>(src + lo + (slice_first + k) * part, dst + k * slice_stride_units + lo / nslices, part);
         __syncthreads();
         if (tid == 0) {
             const int old = __hip_atomic_fetch_add(MM + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -87,10 +123,10 @@ __global__ void __launch_bounds__(256) wait_consume_kernel(const int* __restrict
     }
 }
 
-__global__ void __launch_bounds__(256) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
-                                                      size_t units, const unsigned short* src_tail,
-                                                      unsigned short* dst_tail, int tail) {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < units; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+__global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                               long long units, const unsigned short* src_tail,
+                                                               unsigned short* dst_tail, int tail) {
+    grid_copy<false>(src, dst, units);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
@@ -173,7 +209,7 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
     if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_wait_consume: buffers must be 16-byte aligned");
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
-    hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(256), 0, stream, cseg, G, MM, (const uint4*)src,
+    hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(kCopyThreads), 0, stream, cseg, G, MM, (const uint4*)src,
                        (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks);
     FO_HIP(hipGetLastError());
     return FO_OK;
@@ -186,11 +222,12 @@ int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream)
     if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_consume: buffers must be 16-byte aligned");
     const size_t units = bytes / 16;
     const int tail = (int)((bytes % 16) / 2);
-    size_t blocks = (units + 255) / 256;
-    if (blocks > 2048) blocks = 2048;
+    const size_t per_block = (size_t)kCopyThreads * kCopyUnroll;
+    size_t blocks = (units + per_block - 1) / per_block;
+    if (blocks > 1024) blocks = 1024;
     if (blocks == 0) blocks = 1;
-    hipLaunchKernelGGL(consume_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint4*)src, (uint4*)dst,
-                       units, (const unsigned short*)((const char*)src + units * 16),
+    hipLaunchKernelGGL(consume_kernel, dim3((unsigned)blocks), dim3(kCopyThreads), 0, stream, (const uint4*)src,
+                       (uint4*)dst, (long long)units, (const unsigned short*)((const char*)src + units * 16),
                        (unsigned short*)((char*)dst + units * 16), tail);
     FO_HIP(hipGetLastError());
     return FO_OK;

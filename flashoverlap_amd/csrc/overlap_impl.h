@@ -53,7 +53,7 @@ class OverlapImpl : public torch::CustomClassHolder {
     // beyond), 1 = one (wait, consume) launch pair per group like the
     // reference's host loop, 2 = one persistent wait+consume kernel.
     void SetConsumerMode(int64_t mode);
-    // Workgroups of the persistent consumer (default 8).
+    // Workgroups of the persistent consumer (default 64).
     void SetConsumerBlocks(int64_t blocks);
 
   private:
@@ -63,7 +63,7 @@ class OverlapImpl : public torch::CustomClassHolder {
     int64_t my_rank_ = 0;
     int64_t my_size_ = 1;
     int64_t consumer_mode_ = 0;
-    int64_t consumer_blocks_ = 8;
+    int64_t consumer_blocks_ = 64;
 
     at::Tensor staging_;
     at::Tensor group_table_;
