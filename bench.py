@@ -42,9 +42,11 @@ NAMES = {
 }
 PEAK_MFMA_TFLOPS = 2516.6   # MI355X dense fp16/bf16: 256 CU x 4096 FLOP/clk x 2.4 GHz
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
-# HBM bytes per signalling-GEMM launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# command (profiles/), scaled by a copy kernel of known size; None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {}
+# Bytes that cross the L2 -> memory interface per signalling-GEMM launch, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of `bench.py --no-overlap` (profiles/gemm_signal_c3_traffic.txt):
+# FETCH_SIZE 344248 KiB x 1.997 (the 64 MiB consumer copy reads as 32821 KiB) + WRITE_SIZE 65600 KiB
+# x 1.000.  None for workloads that have not been measured.
+MEASURED_TRAFFIC_BYTES = {"c3": 771_100_000}
 
 
 def main() -> int:
@@ -57,6 +59,9 @@ def main() -> int:
     ap.add_argument("--kernel-iters", type=int, default=100, help="timed launches per isolated kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline work; 0 skips it")
     ap.add_argument("--consumer-blocks", type=int, default=64)
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="order the consumer behind the GEMM in the timed step (needed under counter collection, "
+                         "which runs one kernel at a time)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build drives one GPU only; run with --gpus 1 "
@@ -135,21 +140,27 @@ def main() -> int:
             capi.check(L.fo_reorder_rmsnorm(code, staging.data_ptr(), gamma.data_ptr(), out.data_ptr(), M, N, BM, BN,
                                             1, RA.data_ptr(), eps, main_stream))
 
-    def step():
+    def step(overlap=True):
         gemm_signal()
+        if not overlap:  # consumer ordered behind the GEMM: the serial reference for the overlap
+            capi.check(L.fo_stream_join(main_stream, comm))
         wait_consume()
         capi.check(L.fo_stream_join(comm, main_stream))
         norm()
 
+    def time_steps(overlap):
+        for _ in range(a.warmup):
+            step(overlap)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            step(overlap)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / a.steps
+
     # ---- whole path: W warm-up steps, then exactly K timed steps -----------------
-    for _ in range(a.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        step()
-    torch.cuda.synchronize()
-    step_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    serial_ms = time_steps(False)
+    step_ms = serial_ms if a.no_overlap else time_steps(True)
     timeouts = C.c_int()
     capi.check(L.fo_wait_timeouts(C.byref(timeouts), 1))
     if timeouts.value:
@@ -157,34 +168,40 @@ def main() -> int:
         return 1
 
     # ---- isolated kernels, HIP events on the launch stream -----------------------
-    def time_kernel(fn, iters, after=None):
-        evs = [(C.c_void_p(), C.c_void_p()) for _ in range(iters)]
-        for s, e in evs:
-            capi.check(L.fo_event_create(C.byref(s)))
-            capi.check(L.fo_event_create(C.byref(e)))
+    def time_kernel(fn, iters):
+        """Average launch duration: `iters` back-to-back launches between one HIP event pair on
+        the launch stream (what a kernel trace reports as the kernel's average), and the
+        shortest single launch out of 10 individually bracketed ones."""
+        e0, e1 = C.c_void_p(), C.c_void_p()
+        capi.check(L.fo_event_create(C.byref(e0)))
+        capi.check(L.fo_event_create(C.byref(e1)))
+        v = C.c_float()
         for _ in range(5):
             fn()
-            if after:
-                after()
         torch.cuda.synchronize()
-        for s, e in evs:
-            capi.check(L.fo_event_record(s, main_stream))
+        capi.check(L.fo_event_record(e0, main_stream))
+        for _ in range(iters):
             fn()
-            capi.check(L.fo_event_record(e, main_stream))
-            if after:
-                after()
+        capi.check(L.fo_event_record(e1, main_stream))
         torch.cuda.synchronize()
-        ms = []
-        for s, e in evs:
-            v = C.c_float()
-            capi.check(L.fo_event_elapsed_ms(s, e, C.byref(v)))
-            ms.append(v.value)
-            capi.check(L.fo_event_destroy(s))
-            capi.check(L.fo_event_destroy(e))
-        return sum(ms) / len(ms), min(ms)
+        capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(v)))
+        avg = v.value / iters
+        best = float("inf")
+        for _ in range(10):
+            capi.check(L.fo_event_record(e0, main_stream))
+            fn()
+            capi.check(L.fo_event_record(e1, main_stream))
+            torch.cuda.synchronize()
+            capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(v)))
+            best = min(best, v.value)
+        capi.check(L.fo_event_destroy(e0))
+        capi.check(L.fo_event_destroy(e1))
+        return avg, best
 
     it = a.kernel_iters
-    sig_ms, sig_min = time_kernel(gemm_signal, it, after=lambda: MM.zero_())
+    # no waiter runs here: the group counters simply accumulate and are cleared afterwards
+    sig_ms, sig_min = time_kernel(gemm_signal, it)
+    MM.zero_()
     pl_ms, pl_min = time_kernel(gemm_plain, it)
     rms_ms, rms_min = time_kernel(norm, it)
     cons_ms, _ = time_kernel(
@@ -232,7 +249,9 @@ def main() -> int:
         "config": {"workload": f"{a.workload}: {NAMES[a.workload]}", "M": M, "N": N, "K": K,
                    "layout_tile": [BM, BN], "tiles": T, "tiles_per_group": w, "groups": G, "world_size": ws,
                    "eps": eps, "consumer": f"persistent wait+consume, {a.consumer_blocks} workgroups",
-                   "step": "signal GEMM || wait+consume -> join -> reorder+RMSNorm"},
+                   "step": ("signal GEMM -> wait+consume -> reorder+RMSNorm (serial)" if a.no_overlap else
+                            "signal GEMM || wait+consume -> join -> reorder+RMSNorm")},
+        "serial_step_ms": round(serial_ms, 5),
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (signalling)", "achieved": round(sig_tf, 2),
                      "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": round(sig_tf / PEAK_MFMA_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload), "avg_us": round(sig_ms * 1e3, 2),

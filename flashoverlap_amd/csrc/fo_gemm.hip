@@ -72,7 +72,7 @@ constexpr int kRowBytes = kBK * 2;  // one panel row in LDS: 128 bytes = 8 chunk
 enum { kPlain = 0, kSignal = 1, kScatter = 2 };
 
 // Tuning knobs (fo_tune): how the epilogue stores C and how it signals.
-int g_store_mode = 0;    // 0 = cached stores, 1 = agent-scope write-through stores (sc1)
+int g_store_mode = 1;    // 0 = cached stores, 1 = agent-scope write-through stores (sc1)
 int g_release_mode = 0;  // 0 = release-ordered atomic, 1 = write-through stores + relaxed atomic (needs store mode 1)
 
 struct GemmParams {

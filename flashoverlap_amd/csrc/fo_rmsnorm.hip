@@ -1,9 +1,13 @@
 // RMSNorm and reorder+RMSNorm for gfx950: one 64-lane wavefront per output row,
 // the whole row held in registers between the sum of squares and the scaling,
 // 128-bit coalesced HBM accesses, a wavefront butterfly for the reduction (no
-// LDS, no barrier).  The reorder variant gathers the row from the
-// tile-permuted GEMM output: 16 consecutive lanes read one 256-byte row
-// segment of a 128-wide tile, so every access is made of whole cache lines.
+// LDS, no barrier); gamma is fetched together with the row so that nothing but
+// arithmetic sits between the last load and the first store.  The reorder
+// variant gathers the row from the tile-permuted GEMM output: 16 consecutive
+// lanes read one 256-byte row segment of a 128-wide tile, so every access is
+// made of whole cache lines.  In the common case (rldn == 1, power-of-two tile,
+// at most 64 tiles per row) each lane fetches one RA entry and the lanes
+// exchange them, so the gather costs one small load instead of one per chunk.
 //
 // Arithmetic follows src/rmsnorm/rmsnorm.cuh:62-115 of the reference: fp32 sum
 // of squares, scale = rsqrt(sum/dim + eps), the scaled value rounded to the
@@ -32,30 +36,55 @@ struct Vec8<__bf16> {
 
 constexpr int kRowsPerBlock = 4;  // one wavefront per row
 
+enum { kNormPlain = 0, kNormGather = 1, kNormGatherFast = 2 };
+
+struct NormParams {
+    int bs, dim, BM, BN, rldn;
+    int log_bm, log_bn;  // kNormGatherFast only
+    float eps;
+};
+
 // CH = 16-byte chunks per lane (dim <= CH * 512).
-template <typename T, int CH, bool REORDER>
+template <typename T, int CH, int MODE>
 __global__ void __launch_bounds__(256) rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
-                                                      T* __restrict__ out, int bs, int dim, int BM, int BN,
-                                                      int rldn, const int* __restrict__ RA, float eps) {
+                                                      T* __restrict__ out, const int* __restrict__ RA,
+                                                      const NormParams p) {
     using vec = typename Vec8<T>::type;
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
-    if (row >= bs) return;
+    if (row >= p.bs) return;
 
+    const int dim = p.dim;
     const int nchunk = dim >> 3;
-    vec xv[CH];
-    if constexpr (REORDER) {
-        const int ldn = dim / BN;
-        const int tile_row = (row / BM) * ldn;
-        const int in_row = row % BM;
-        const int ld = rldn * BN;
+    vec xv[CH], gv[CH];
+    if constexpr (MODE == kNormGatherFast) {
+        // tiles of this row: RA[tile_row .. tile_row + ldn), ldn <= 64: one entry per lane
+        const int ldn = dim >> p.log_bn;
+        const int tile_row = (row >> p.log_bm) * ldn;
+        const int in_row = row & (p.BM - 1);
+        const int mine = RA[tile_row + (lane < ldn ? lane : 0)];
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+            const int c = k * 64 + lane;
+            const int j = c << 3;
+            const int s = __shfl(mine, (j >> p.log_bn) & 63, 64);  // all lanes take part in the exchange
+            if (c < nchunk) {
+                const size_t src = ((((size_t)s << p.log_bm) + in_row) << p.log_bn) + (j & (p.BN - 1));
+                xv[k] = *(const vec*)(x + src);
+            }
+        }
+    } else if constexpr (MODE == kNormGather) {
+        const int ldn = dim / p.BN;
+        const int tile_row = (row / p.BM) * ldn;
+        const int in_row = row % p.BM;
+        const int ld = p.rldn * p.BN;
 #pragma unroll
         for (int k = 0; k < CH; ++k) {
             const int c = k * 64 + lane;
             if (c < nchunk) {
                 const int j = c << 3;
-                const int s = RA[tile_row + j / BN];
-                const size_t src = (size_t)((s / rldn) * BM + in_row) * ld + (s % rldn) * BN + j % BN;
+                const int s = RA[tile_row + j / p.BN];
+                const size_t src = (size_t)((s / p.rldn) * p.BM + in_row) * ld + (s % p.rldn) * p.BN + j % p.BN;
                 xv[k] = *(const vec*)(x + src);
             }
         }
@@ -66,6 +95,11 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const T* __restrict__ x, c
             const int c = k * 64 + lane;
             if (c < nchunk) xv[k] = *(const vec*)(xr + (c << 3));
         }
+    }
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+        const int c = k * 64 + lane;
+        if (c < nchunk) gv[k] = *(const vec*)(gamma + (c << 3));
     }
 
     float ss = 0.f;
@@ -81,33 +115,39 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const T* __restrict__ x, c
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
-    const float scale = rsqrtf(ss / (float)dim + eps);
+    const float scale = rsqrtf(ss / (float)dim + p.eps);
 
     T* orow = out + (size_t)row * dim;
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
         const int c = k * 64 + lane;
         if (c < nchunk) {
-            const vec g = *(const vec*)(gamma + (c << 3));
             vec o;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const T y = (T)((float)xv[k][e] * scale);
-                o[e] = (T)((float)y * (float)g[e]);
+                o[e] = (T)((float)y * (float)gv[k][e]);
             }
             *(vec*)(orow + (c << 3)) = o;
         }
     }
 }
 
-template <typename T, bool REORDER>
-static int launch_t(const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN, int rldn,
-                    const int* RA, float eps, hipStream_t stream) {
-    const int ch = (dim / 8 + 63) / 64;
-    const dim3 grid((bs + kRowsPerBlock - 1) / kRowsPerBlock), block(64 * kRowsPerBlock);
-#define FO_RMS_CASE(CH)                                                                                   \
-    hipLaunchKernelGGL((rmsnorm_kernel<T, CH, REORDER>), grid, block, 0, stream, (const T*)x, (const T*)gamma, \
-                       (T*)out, bs, dim, BM, BN, rldn, RA, eps)
+static int log2_exact(int v) {
+    if (v <= 0 || (v & (v - 1))) return -1;
+    int l = 0;
+    while ((1 << l) < v) ++l;
+    return l;
+}
+
+template <typename T, int MODE>
+static int launch_t(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p,
+                    hipStream_t stream) {
+    const int ch = (p.dim / 8 + 63) / 64;
+    const dim3 grid((p.bs + kRowsPerBlock - 1) / kRowsPerBlock), block(64 * kRowsPerBlock);
+#define FO_RMS_CASE(CH)                                                                                       \
+    hipLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, 0, stream, (const T*)x, (const T*)gamma, \
+                       (T*)out, RA, p)
     if (ch <= 1) FO_RMS_CASE(1);
     else if (ch <= 2) FO_RMS_CASE(2);
     else if (ch <= 4) FO_RMS_CASE(4);
@@ -117,6 +157,14 @@ static int launch_t(const void* x, const void* gamma, void* out, int bs, int dim
 #undef FO_RMS_CASE
     FO_HIP(hipGetLastError());
     return FO_OK;
+}
+
+template <typename T>
+static int launch_dtype(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p,
+                        hipStream_t stream) {
+    if (!RA) return launch_t<T, kNormPlain>(x, gamma, out, RA, p, stream);
+    if (p.log_bm >= 0) return launch_t<T, kNormGatherFast>(x, gamma, out, RA, p, stream);
+    return launch_t<T, kNormGather>(x, gamma, out, RA, p, stream);
 }
 
 int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
@@ -130,17 +178,19 @@ int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int b
     if (dim % 8) return fail(FO_ERR_SHAPE, "%s: dim=%d not a multiple of 8", who, dim);
     if (dim > 32 * 512) return fail(FO_ERR_LIMIT, "%s: dim=%d above the 16384 a wavefront keeps in registers", who, dim);
     if (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)out) & 15) return fail(FO_ERR_ARG, "%s: buffers must be 16-byte aligned", who);
+    NormParams p{bs, dim, BM, BN, rldn, -1, -1, eps};
     if (reorder) {
         if (BM <= 0 || BN <= 0 || rldn <= 0) return fail(FO_ERR_ARG, "%s: BM=%d BN=%d rldn=%d", who, BM, BN, rldn);
         if (BN % 8 || dim % BN) return fail(FO_ERR_SHAPE, "%s: BN=%d must be a multiple of 8 that divides dim=%d", who, BN, dim);
         if (bs % BM) return fail(FO_ERR_SHAPE, "%s: bs=%d not a multiple of BM=%d", who, bs, BM);
         if (((long long)(bs / BM) * (dim / BN)) % rldn) return fail(FO_ERR_SHAPE, "%s: rldn=%d must divide the tile count", who, rldn);
+        if (rldn == 1 && dim / BN <= 64 && log2_exact(BM) >= 0 && log2_exact(BN) >= 0) {
+            p.log_bm = log2_exact(BM);
+            p.log_bn = log2_exact(BN);
+        }
     }
-    if (dtype == FO_F16)
-        return reorder ? launch_t<_Float16, true>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream)
-                       : launch_t<_Float16, false>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream);
-    return reorder ? launch_t<__bf16, true>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream)
-                   : launch_t<__bf16, false>(x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, stream);
+    if (dtype == FO_F16) return launch_dtype<_Float16>(x, gamma, out, RA, p, stream);
+    return launch_dtype<__bf16>(x, gamma, out, RA, p, stream);
 }
 
 }  // namespace fo

@@ -106,8 +106,9 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host);
 
 /* Process-wide tuning knobs of the GEMM epilogue, for measurement; no
  * counterpart in the reference.  Results are identical for every setting.
- *   "store_mode"   0: cached tile stores (default); 1: agent-scope
- *                  write-through tile stores.
+ *   "store_mode"   0: cached tile stores; 1: agent-scope write-through tile
+ *                  stores (default: the release then finds no dirty lines to
+ *                  write back).
  *   "release_mode" 0: release-ordered signal atomic (default); 1: write-through
  *                  tile stores, wait for their acknowledgement, relaxed atomic. */
 int fo_tune(const char* key, int value);
