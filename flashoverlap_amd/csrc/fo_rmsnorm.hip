@@ -34,7 +34,7 @@ struct Vec8<__bf16> {
     using type = bf16x8;
 };
 
-constexpr int kRowsPerBlock = 4;  // one wavefront per row
+constexpr int kRowsPerBlock = 1;  // one wavefront per row, one row per workgroup
 
 enum { kNormPlain = 0, kNormGather = 1, kNormGatherFast = 2 };
 
@@ -46,7 +46,7 @@ struct NormParams {
 
 // CH = 16-byte chunks per lane (dim <= CH * 512).
 template <typename T, int CH, int MODE>
-__global__ void __launch_bounds__(256) rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
+__global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
                                                       T* __restrict__ out, const int* __restrict__ RA,
                                                       const NormParams p) {
     using vec = typename Vec8<T>::type;
@@ -116,6 +116,11 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const T* __restrict__ x, c
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
     const float scale = rsqrtf(ss / (float)dim + p.eps);
+    // The row stays packed in its 16-bit form across the reduction; without this
+    // the fp32 copies made for the sum of squares are kept alive too, which
+    // doubles the register footprint and halves the waves per SIMD.
+#pragma unroll
+    for (int k = 0; k < CH; ++k) asm volatile("" : "+v"(xv[k]));
 
     T* orow = out + (size_t)row * dim;
 #pragma unroll
