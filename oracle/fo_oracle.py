@@ -378,3 +378,60 @@ def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
 
 def max_abs(a: torch.Tensor, b: torch.Tensor) -> float:
     return float((a.double() - b.double()).abs().max())
+
+
+# --------------------------------------------------------------------------
+# tuner
+# --------------------------------------------------------------------------
+
+
+def vote_hint_literal(samples, wSize: int):
+    """Statement-by-statement twin of the majority vote in tune/search.py:218-263
+    (plain loops; torch.mode's tie rule = smallest value)."""
+    n = len(samples)
+    TileNum = len(samples[0])
+    WaveNum = div_up(TileNum, wSize)
+    tile_wave = [[min(samples[i][t] // wSize, WaveNum - 1) for t in range(TileNum)] for i in range(n)]
+    tile_modes, mode_counts = [], []
+    for ti in range(TileNum):
+        col = [tile_wave[i][ti] for i in range(n)]
+        best = max(set(col), key=lambda v: (col.count(v), -v))
+        tile_modes.append(best)
+        mode_counts.append(col.count(best))
+    wave_tiles = {w: [] for w in range(WaveNum)}
+    for ti in range(TileNum):
+        wave_tiles[tile_modes[ti]].append((mode_counts[ti], ti))
+    for w in wave_tiles:
+        wave_tiles[w].sort(reverse=True)
+    unassigned = []
+    assigned = {w: [] for w in range(WaveNum)}
+    for w in range(WaveNum):
+        target = wSize if w < WaveNum - 1 else TileNum - w * wSize
+        tiles = wave_tiles[w]
+        assigned[w] = [t[1] for t in tiles[:target]]
+        unassigned.extend([t[1] for t in tiles[target:]])
+    for w in range(WaveNum):
+        target = wSize if w < WaveNum - 1 else TileNum - w * wSize
+        while len(assigned[w]) < target and unassigned:
+            assigned[w].append(unassigned.pop())
+    hint = []
+    for w in range(WaveNum):
+        target = wSize if w < WaveNum - 1 else TileNum - w * wSize
+        if len(assigned[w]) < target:
+            return False, []
+        hint.extend(assigned[w])
+    return True, hint
+
+
+def predict_latency_literal(gemm_dur, comm_ms, gp, wave_size, tile_num, tile_bytes):
+    """Pipeline recurrence of tune/search.py:316-344 without the reference's
+    rescaling for compute units set aside for the collective."""
+    if len(gp) == 1:
+        return comm_ms(gp[0] * tile_bytes) + gemm_dur
+    wave_num = div_up(tile_num, wave_size)
+    acc_comm = acc_comp = 0.0
+    for i in range(len(gp)):
+        comm = 0.0 if i == 0 else comm_ms(gp[i - 1] * tile_bytes)
+        acc_comm = max(acc_comp, acc_comm) + comm
+        acc_comp += gemm_dur / wave_num * div_up(gp[i], wave_size)
+    return max(acc_comp, acc_comm) + comm_ms(gp[-1] * tile_bytes)
