@@ -131,11 +131,9 @@ def main() -> int:
                                      ws, 0, ws, (M * N // ws) if ws > 1 else 0, None, a.consumer_blocks, comm))
 
     def norm():
-        if ws > 1:  # every rank slice is a layout with tile height BM/ws
-            for k in range(ws):
-                capi.check(L.fo_reorder_rmsnorm(code, staging.data_ptr() + 2 * k * (M * N // ws), gamma.data_ptr(),
-                                                out.data_ptr() + 2 * k * (M * N // ws), M // ws, N, BM // ws, BN, 1,
-                                                RA.data_ptr(), eps, main_stream))
+        if ws > 1:  # every rank slice is a layout with tile height BM/ws: ws problems, one launch
+            capi.check(L.fo_reorder_rmsnorm_batched(code, staging.data_ptr(), gamma.data_ptr(), out.data_ptr(), ws,
+                                                    M // ws, N, BM // ws, BN, 1, RA.data_ptr(), eps, main_stream))
         else:
             capi.check(L.fo_reorder_rmsnorm(code, staging.data_ptr(), gamma.data_ptr(), out.data_ptr(), M, N, BM, BN,
                                             1, RA.data_ptr(), eps, main_stream))

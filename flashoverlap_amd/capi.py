@@ -35,6 +35,7 @@ SIGNATURES = {
     "fo_wait_timeouts": (_i, [_ip, _i]),
     "fo_consume": (_i, [_vp, _vp, _sz, _vp]),
     "fo_reorder_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
+    "fo_reorder_rmsnorm_batched": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "fo_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _f, _vp]),
     "fo_stream_create": (_i, [C.POINTER(_vp)]),
     "fo_stream_destroy": (_i, [_vp]),
@@ -72,6 +73,10 @@ def lib() -> C.CDLL:
             fn = getattr(handle, name)
             fn.restype, fn.argtypes = res, args
         _lib = handle
+        # FO_TUNE="knob=value,knob=value" applies fo_tune settings at load time
+        for item in filter(None, os.environ.get("FO_TUNE", "").split(",")):
+            key, _, value = item.partition("=")
+            check(handle.fo_tune(key.strip().encode(), int(value)))
     return _lib
 
 

@@ -112,11 +112,17 @@ int fo_consume(const void* src, void* dst, size_t bytes, void* stream) {
 int fo_reorder_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
                        int rldn, const int* RA, float eps, void* stream) {
     if (!RA) return fail(FO_ERR_ARG, "fo_reorder_rmsnorm: null RA");
-    return launch_rmsnorm(dtype, x, gamma, out, bs, dim, BM, BN, rldn, RA, eps, (hipStream_t)stream);
+    return launch_rmsnorm(dtype, x, gamma, out, 1, bs, dim, BM, BN, rldn, RA, eps, (hipStream_t)stream);
+}
+
+int fo_reorder_rmsnorm_batched(int dtype, const void* x, const void* gamma, void* out, int nbatch, int bs, int dim,
+                               int BM, int BN, int rldn, const int* RA, float eps, void* stream) {
+    if (!RA) return fail(FO_ERR_ARG, "fo_reorder_rmsnorm_batched: null RA");
+    return launch_rmsnorm(dtype, x, gamma, out, nbatch, bs, dim, BM, BN, rldn, RA, eps, (hipStream_t)stream);
 }
 
 int fo_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, float eps, void* stream) {
-    return launch_rmsnorm(dtype, x, gamma, out, bs, dim, 0, 0, 0, nullptr, eps, (hipStream_t)stream);
+    return launch_rmsnorm(dtype, x, gamma, out, 1, bs, dim, 0, 0, 0, nullptr, eps, (hipStream_t)stream);
 }
 
 int fo_stream_create(void** stream) {

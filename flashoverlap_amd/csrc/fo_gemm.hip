@@ -185,6 +185,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
             sig_group = p.gtable ? p.gtable[sig_slot] : scan_group(p.cseg, sig_slot);
         }
     }
+    // Scatter: the remapped destination rows of this quadrant, one or two per
+    // lane, fetched now and handed round between the lanes in the epilogue.
+    [[maybe_unused]] int re_lo = 0, re_hi = 0;
+    if constexpr (MODE == kScatter) {
+        re_lo = p.RE[row0 + (lane < WT ? lane : 0)];
+        if constexpr (WT > 64) re_hi = p.RE[row0 + 64 + lane];
+    }
 
     // ---- HBM -> LDS copy addressing ------------------------------------------
     // One copy instruction moves 1 KiB = 8 panel rows of 128 bytes: lane l's 16
@@ -374,7 +381,10 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
             const int r = c / ROWCH, cc = c % ROWCH;
             const u32x4 v = *(const u32x4*)(ep + r * PITCH + cc * 16);
             int row = row0 + 32 * i + r;
-            if constexpr (MODE == kScatter) row = p.RE[row];
+            if constexpr (MODE == kScatter) {
+                const int q_row = 32 * i + r;   // row within the quadrant: held by lane q_row % 64
+                row = __shfl((WT > 64 && i >= 2) ? re_hi : re_lo, q_row & 63, 64);
+            }
             const size_t off = (size_t)row * ld + col0 + cc * 8;
             if constexpr (STORE == 1)
                 __builtin_amdgcn_raw_buffer_store_b128(v, drsrc, (int)(off * 2), 0, 16);  // sc1: write-through

@@ -40,7 +40,7 @@ int set_wait_timeout_ms(int ms);
 int wait_timeouts(int* count, int reset);
 
 // fo_rmsnorm.hip
-int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
-                   int rldn, const int* RA, float eps, hipStream_t stream);
+int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int nbatch, int bs, int dim, int BM,
+                   int BN, int rldn, const int* RA, float eps, hipStream_t stream);
 
 }  // namespace fo

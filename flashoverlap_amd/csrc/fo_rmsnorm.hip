@@ -46,13 +46,16 @@ struct NormParams {
 
 // CH = 16-byte chunks per lane (dim <= CH * 512).
 template <typename T, int CH, int MODE>
-__global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ gamma,
-                                                      T* __restrict__ out, const int* __restrict__ RA,
+__global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __restrict__ x0, const T* __restrict__ gamma,
+                                                      T* __restrict__ out0, const int* __restrict__ RA,
                                                       const NormParams p) {
     using vec = typename Vec8<T>::type;
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
     if (row >= p.bs) return;
+    // blockIdx.y selects one of several independent [bs, dim] problems laid out back to back
+    const T* __restrict__ x = x0 + (size_t)blockIdx.y * p.bs * p.dim;
+    T* __restrict__ out = out0 + (size_t)blockIdx.y * p.bs * p.dim;
 
     const int dim = p.dim;
     const int nchunk = dim >> 3;
@@ -146,10 +149,10 @@ static int log2_exact(int v) {
 }
 
 template <typename T, int MODE>
-static int launch_t(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p,
+static int launch_t(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p, int nbatch,
                     hipStream_t stream) {
     const int ch = (p.dim / 8 + 63) / 64;
-    const dim3 grid((p.bs + kRowsPerBlock - 1) / kRowsPerBlock), block(64 * kRowsPerBlock);
+    const dim3 grid((p.bs + kRowsPerBlock - 1) / kRowsPerBlock, nbatch), block(64 * kRowsPerBlock);
 #define FO_RMS_CASE(CH)                                                                                       \
     hipLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, 0, stream, (const T*)x, (const T*)gamma, \
                        (T*)out, RA, p)
@@ -165,19 +168,20 @@ static int launch_t(const void* x, const void* gamma, void* out, const int* RA, 
 }
 
 template <typename T>
-static int launch_dtype(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p,
+static int launch_dtype(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p, int nbatch,
                         hipStream_t stream) {
-    if (!RA) return launch_t<T, kNormPlain>(x, gamma, out, RA, p, stream);
-    if (p.log_bm >= 0) return launch_t<T, kNormGatherFast>(x, gamma, out, RA, p, stream);
-    return launch_t<T, kNormGather>(x, gamma, out, RA, p, stream);
+    if (!RA) return launch_t<T, kNormPlain>(x, gamma, out, RA, p, nbatch, stream);
+    if (p.log_bm >= 0) return launch_t<T, kNormGatherFast>(x, gamma, out, RA, p, nbatch, stream);
+    return launch_t<T, kNormGather>(x, gamma, out, RA, p, nbatch, stream);
 }
 
-int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
-                   int rldn, const int* RA, float eps, hipStream_t stream) {
+int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int nbatch, int bs, int dim, int BM,
+                   int BN, int rldn, const int* RA, float eps, hipStream_t stream) {
     const bool reorder = RA != nullptr;
     const char* who = reorder ? "fo_reorder_rmsnorm" : "fo_rmsnorm";
     if (dtype != FO_F16 && dtype != FO_BF16) return fail(FO_ERR_ARG, "%s: dtype %d not fp16/bf16", who, dtype);
-    if (bs == 0) return FO_OK;
+    if (bs == 0 || nbatch == 0) return FO_OK;
+    if (nbatch < 0 || nbatch > 65535) return fail(FO_ERR_LIMIT, "%s: %d batches outside 0..65535", who, nbatch);
     if (!x || !gamma || !out) return fail(FO_ERR_ARG, "%s: null buffer", who);
     if (bs < 0 || dim <= 0) return fail(FO_ERR_SHAPE, "%s: bs=%d dim=%d", who, bs, dim);
     if (dim % 8) return fail(FO_ERR_SHAPE, "%s: dim=%d not a multiple of 8", who, dim);
@@ -194,8 +198,8 @@ int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int b
             p.log_bn = log2_exact(BN);
         }
     }
-    if (dtype == FO_F16) return launch_dtype<_Float16>(x, gamma, out, RA, p, stream);
-    return launch_dtype<__bf16>(x, gamma, out, RA, p, stream);
+    if (dtype == FO_F16) return launch_dtype<_Float16>(x, gamma, out, RA, p, nbatch, stream);
+    return launch_dtype<__bf16>(x, gamma, out, RA, p, nbatch, stream);
 }
 
 }  // namespace fo

@@ -162,6 +162,16 @@ int fo_reorder_rmsnorm(int dtype, const void* x, const void* gamma, void* out,
                        int bs, int dim, int BM, int BN, int rldn, const int* RA,
                        float eps, void* stream);
 
+/* nbatch independent reorder+RMSNorm problems in one launch: x and out hold
+ * nbatch consecutive [bs, dim] blocks that all use the same RA, BM, BN.  This is
+ * the shape of the ReduceScatter receive buffers of all ranks side by side
+ * (each a tile-permuted layout with tile height BM/world_size,
+ * example/correctness_rs.py:107-108 builds one of them per rank); no counterpart
+ * in the reference, where a process only ever holds its own rank's buffer. */
+int fo_reorder_rmsnorm_batched(int dtype, const void* x, const void* gamma, void* out,
+                               int nbatch, int bs, int dim, int BM, int BN, int rldn,
+                               const int* RA, float eps, void* stream);
+
 /* Plain row RMSNorm.  Replaces launch_rmsnorm_kernel
  * (src/rmsnorm/rmsnorm_launch.h:5, src/rmsnorm/rmsnorm.cuh:12-57). */
 int fo_rmsnorm(int dtype, const void* x, const void* gamma, void* out,
