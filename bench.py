@@ -7,11 +7,14 @@ second stream releasing each finished group into the staging buffer, an event
 join, then reorder+RMSNorm on the staging buffer.
 
 Prints ONE JSON line.  `value` is 2*M*N*K divided by the whole step time.  The
-roofline object is for the dominant kernel (the signalling GEMM), timed live
-with HIP events on its own stream; the same run also times the plain-GEMM twin
-(signal overhead), reorder+RMSNorm (HBM roofline) and the consumer copy, and a
-CPU baseline (the oracle's fp32 matmul + RMSNorm on the host cores) on a
-bounded sample of the same workload.
+roofline object is for the dominant kernel (the signalling GEMM) as it ran
+inside the timed steps, from HIP events around every launch on its own stream.
+The same run also times, back to back and on their own, the signalling GEMM
+and its plain twin (signal overhead), reorder+RMSNorm (HBM roofline) and the
+consumer copy, the serial (non-overlapped) step, and a CPU baseline (the
+oracle's fp32 matmul + RMSNorm on the host cores) on a bounded sample of the
+same workload.  Launch order: W+K serial steps, W+K overlapped steps, then the
+isolated kernels (5 warm-up + --kernel-iters + 10 launches each).
 """
 from __future__ import annotations
 
@@ -43,10 +46,10 @@ NAMES = {
 PEAK_MFMA_TFLOPS = 2516.6   # MI355X dense fp16/bf16: 256 CU x 4096 FLOP/clk x 2.4 GHz
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # Bytes that cross the L2 -> memory interface per signalling-GEMM launch, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs of `bench.py --no-overlap` (profiles/gemm_signal_c3_traffic.txt):
-# FETCH_SIZE 344248 KiB x 1.997 (the 64 MiB consumer copy reads as 32821 KiB) + WRITE_SIZE 65600 KiB
+# FETCH_SIZE / WRITE_SIZE runs of `bench.py --no-overlap` (profiles/gemm_signal_c3_counters.txt):
+# FETCH_SIZE 344245 KiB x 1.999 (the 64 MiB consumer copy reads as 32786.5 KiB) + WRITE_SIZE 65600 KiB
 # x 1.000.  None for workloads that have not been measured.
-MEASURED_TRAFFIC_BYTES = {"c3": 771_100_000}
+MEASURED_TRAFFIC_BYTES = {"c3": 771_800_000}
 
 
 def main() -> int:
@@ -138,8 +141,12 @@ def main() -> int:
             capi.check(L.fo_reorder_rmsnorm(code, staging.data_ptr(), gamma.data_ptr(), out.data_ptr(), M, N, BM, BN,
                                             1, RA.data_ptr(), eps, main_stream))
 
-    def step(overlap=True):
+    def step(overlap=True, ev=None):
+        if ev:
+            capi.check(L.fo_event_record(ev[0], main_stream))
         gemm_signal()
+        if ev:
+            capi.check(L.fo_event_record(ev[1], main_stream))
         if not overlap:  # consumer ordered behind the GEMM: the serial reference for the overlap
             capi.check(L.fo_stream_join(main_stream, comm))
         wait_consume()
@@ -147,18 +154,33 @@ def main() -> int:
         norm()
 
     def time_steps(overlap):
+        """Wall time per step, and the signalling GEMM's own duration inside those same
+        steps (one HIP event pair per step on the GEMM's stream)."""
+        evs = []
+        for _ in range(a.steps):
+            e0, e1 = C.c_void_p(), C.c_void_p()
+            capi.check(L.fo_event_create(C.byref(e0)))
+            capi.check(L.fo_event_create(C.byref(e1)))
+            evs.append((e0, e1))
         for _ in range(a.warmup):
             step(overlap)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(a.steps):
-            step(overlap)
+        for ev in evs:
+            step(overlap, ev)
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / a.steps
+        wall = (time.perf_counter() - t0) * 1e3 / a.steps
+        v, tot = C.c_float(), 0.0
+        for e0, e1 in evs:
+            capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(v)))
+            tot += v.value
+            capi.check(L.fo_event_destroy(e0))
+            capi.check(L.fo_event_destroy(e1))
+        return wall, tot / a.steps
 
     # ---- whole path: W warm-up steps, then exactly K timed steps -----------------
-    serial_ms = time_steps(False)
-    step_ms = serial_ms if a.no_overlap else time_steps(True)
+    serial_ms, serial_gemm_ms = time_steps(False)
+    step_ms, step_gemm_ms = (serial_ms, serial_gemm_ms) if a.no_overlap else time_steps(True)
     timeouts = C.c_int()
     capi.check(L.fo_wait_timeouts(C.byref(timeouts), 1))
     if timeouts.value:
@@ -250,10 +272,19 @@ def main() -> int:
                    "step": ("signal GEMM -> wait+consume -> reorder+RMSNorm (serial)" if a.no_overlap else
                             "signal GEMM || wait+consume -> join -> reorder+RMSNorm")},
         "serial_step_ms": round(serial_ms, 5),
-        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (signalling)", "achieved": round(sig_tf, 2),
-                     "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": round(sig_tf / PEAK_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload), "avg_us": round(sig_ms * 1e3, 2),
-                     "min_us": round(sig_min * 1e3, 2), "launches": it},
+        # the dominant kernel as it ran inside the timed steps (consumer on the other stream, the
+        # copy and the norm of the previous step in between launches)
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel (signalling), inside the timed steps",
+                     "achieved": round(flops / step_gemm_ms / 1e9, 2), "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / step_gemm_ms / 1e9 / PEAK_MFMA_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload), "avg_us": round(step_gemm_ms * 1e3, 2),
+                     "launches": a.steps},
+        "gemm_signal_serial_step": {"achieved": round(flops / serial_gemm_ms / 1e9, 2), "unit": "TFLOP/s",
+                                    "avg_us": round(serial_gemm_ms * 1e3, 2)},
+        # the same kernel launched back to back on its own (A and B stay in the 256 MB Infinity Cache)
+        "gemm_signal_isolated": {"achieved": round(sig_tf, 2), "unit": "TFLOP/s",
+                                 "frac": round(sig_tf / PEAK_MFMA_TFLOPS, 4), "avg_us": round(sig_ms * 1e3, 2),
+                                 "min_us": round(sig_min * 1e3, 2), "launches": it},
         "cpu_baseline": cpu,
         "gemm_plain": {"achieved": round(pl_tf, 2), "unit": "TFLOP/s", "frac": round(pl_tf / PEAK_MFMA_TFLOPS, 4),
                        "avg_us": round(pl_ms * 1e3, 2), "min_us": round(pl_min * 1e3, 2)},
