@@ -2,9 +2,10 @@
 """Benchmark of the single-GPU hot path on one MI355X.
 
 A step is one pass of the path over one synthetic batch, inputs resident in HBM:
-signalling GEMM on the caller's stream, the persistent wait+consume kernel on a
-second stream releasing each finished group into the staging buffer, an event
-join, then reorder+RMSNorm on the staging buffer.
+signalling GEMM on the caller's stream, on a second stream a wait kernel and a
+consumer copy per group (or one persistent wait+consume kernel) releasing each
+finished group into the staging buffer, an event join, then reorder+RMSNorm on
+the staging buffer.
 
 Prints ONE JSON line.  `value` is 2*M*N*K divided by the whole step time.  The
 roofline object is for the dominant kernel (the signalling GEMM) as it ran
@@ -28,13 +29,17 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# BASELINE.json configs[2..4] plus the small ones; (dtype, M, N, K, tiles per group, world size, eps, a_std, b_std)
+# BASELINE.json configs; (dtype, M, N, K, tiles per group, world size, eps, a_std, b_std).  A hardware
+# wave of the GEMM kernel is 256 workgroups x 4 layout tiles = 1024 tiles of 128x128 (W); the tiles of
+# one wave finish together, so groups are whole waves: c3 one wave per group, c4 two ("group size 2").
+# c1 and c2 fit in one wave and keep the tile-count reading of their group sizes (4 and 256 tiles).
+TILES_PER_WAVE = 1024
 WORKLOADS = {
     "c1": ("fp16", 1024, 1024, 1024, 4, 1, 1e-6, None, None),
     "c2": ("fp16", 4096, 4096, 4096, 256, 1, 1e-5, None, None),
-    "c3": ("bf16", 8192, 4096, 7168, 256, 1, 1e-5, 1.0, 0.02),
-    "c4": ("bf16", 16384, 8192, 1024, 512, 1, 1e-5, None, None),
-    "c5": ("bf16", 8192, 8192, 3584, 256, 8, 1e-5, None, None),
+    "c3": ("bf16", 8192, 4096, 7168, TILES_PER_WAVE, 1, 1e-5, 1.0, 0.02),
+    "c4": ("bf16", 16384, 8192, 1024, 2 * TILES_PER_WAVE, 1, 1e-5, None, None),
+    "c5": ("bf16", 8192, 8192, 3584, TILES_PER_WAVE, 8, 1e-5, None, None),
 }
 NAMES = {
     "c1": "fp16 1024^3 plumbing shape",
@@ -61,7 +66,8 @@ def main() -> int:
     ap.add_argument("--group-tiles", type=int, default=0, help="tiles per signal group (0 = workload default)")
     ap.add_argument("--kernel-iters", type=int, default=100, help="timed launches per isolated kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline work; 0 skips it")
-    ap.add_argument("--consumer-blocks", type=int, default=64)
+    ap.add_argument("--consumer-blocks", type=int, default=64, help="workgroups of the persistent consumer")
+    ap.add_argument("--consumer", default="auto", choices=["auto", "per_group", "persistent"])
     ap.add_argument("--no-overlap", action="store_true",
                     help="order the consumer behind the GEMM in the timed step (needed under counter collection, "
                          "which runs one kernel at a time)")
@@ -129,9 +135,25 @@ def main() -> int:
     def gemm_plain():
         capi.check(L.fo_gemm(code, algo, M, N, K, A.data_ptr(), B.data_ptr(), Cn.data_ptr(), main_stream))
 
+    # Same rule as OverlapImpl: up to 32 groups the reference's structure (one wait kernel and one
+    # consumer launch per group, src/overlap_impl.cu:257-265), beyond that one persistent kernel.
+    per_group = a.consumer == "per_group" or (a.consumer == "auto" and G <= 32)
+
     def wait_consume():
-        capi.check(L.fo_wait_consume(cseg_d.data_ptr(), G, MM.data_ptr(), Cp.data_ptr(), staging.data_ptr(), BM * BN,
-                                     ws, 0, ws, (M * N // ws) if ws > 1 else 0, None, a.consumer_blocks, comm))
+        if not per_group:
+            capi.check(L.fo_wait_consume(cseg_d.data_ptr(), G, MM.data_ptr(), Cp.data_ptr(), staging.data_ptr(),
+                                         BM * BN, ws, 0, ws, (M * N // ws) if ws > 1 else 0, None,
+                                         a.consumer_blocks, comm))
+            return
+        acc = 0
+        for g, n in enumerate(cseg):
+            capi.check(L.fo_wait(n, MM.data_ptr() + 4 * g, comm))
+            elems = n * BM * BN
+            part = elems // ws
+            for k in range(ws):  # ws > 1: slice k of the group goes to rank k's receive buffer
+                capi.check(L.fo_consume(Cp.data_ptr() + 2 * (acc + k * part),
+                                        staging.data_ptr() + 2 * (k * (M * N // ws) + acc // ws), 2 * part, comm))
+            acc += elems
 
     def norm():
         if ws > 1:  # every rank slice is a layout with tile height BM/ws: ws problems, one launch
@@ -267,8 +289,9 @@ def main() -> int:
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(step_ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dts, "data": "synthetic",
         "config": {"workload": f"{a.workload}: {NAMES[a.workload]}", "M": M, "N": N, "K": K,
-                   "layout_tile": [BM, BN], "tiles": T, "tiles_per_group": w, "groups": G, "world_size": ws,
-                   "eps": eps, "consumer": f"persistent wait+consume, {a.consumer_blocks} workgroups",
+                   "layout_tile": [BM, BN], "tiles": T, "tiles_per_wave": TILES_PER_WAVE, "tiles_per_group": w, "groups": G, "world_size": ws,
+                   "eps": eps, "consumer": ("one wait kernel + one copy launch per group" if per_group else
+                                f"persistent wait+consume, {a.consumer_blocks} workgroups"),
                    "step": ("signal GEMM -> wait+consume -> reorder+RMSNorm (serial)" if a.no_overlap else
                             "signal GEMM || wait+consume -> join -> reorder+RMSNorm")},
         "serial_step_ms": round(serial_ms, 5),
