@@ -13,10 +13,11 @@
 // half-line requests cost a quarter of the throughput.  The 16-byte chunks of a
 // row are XOR-swizzled by row so the ds_read_b128 fragment reads are
 // bank-conflict free.  A k-step of 64 is four quarter steps of 16 MFMAs each;
-// fragments are double-buffered in registers, so while one quarter's MFMAs
-// run the next quarter's fragments (in the last quarter: the next panel's) are
-// already being read.  The copies of panel p+2 start as soon as panel p has
-// been read for the last time, and there is one workgroup barrier per k-step.
+// the fragments of all four are read during the first two, so while one
+// quarter's MFMAs run the fragments of the next are already in registers, and
+// the workgroup barrier that hands the panel's buffer to the copies of panel
+// p+2 sits in the middle of the k-step, two quarter steps before the last MFMA
+// on that panel.  There is one barrier per k-step.
 //
 // Epilogue: the quadrant goes through LDS in strips of 32 rows so that every
 // global store instruction writes four whole 256-byte row segments, either to
@@ -245,27 +246,28 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    frag a0[NB], b0[NB], a1[NB], b1[NB];
+    // Fragments of the four quarter steps of a panel (k 0..15, 16..31, 32..47, 48..63).
+    frag fa[4][NB], fb[4][NB];
 
-    auto load_frags = [&](int buf, int kofs, frag(&a)[NB], frag(&b)[NB]) {
-        const unsigned char* base = smem + buf * BUF + kofs;
+    auto load_frags = [&](int buf, int q) {
+        const unsigned char* base = smem + buf * BUF + ko[q];
 #pragma unroll
-        for (int i = 0; i < NB; ++i) a[i] = *(const frag*)(base + a_lane + i * BLK);
+        for (int i = 0; i < NB; ++i) fa[q][i] = *(const frag*)(base + a_lane + i * BLK);
 #pragma unroll
-        for (int j = 0; j < NB; ++j) b[j] = *(const frag*)(base + b_lane + j * BLK);
+        for (int j = 0; j < NB; ++j) fb[q][j] = *(const frag*)(base + b_lane + j * BLK);
     };
     // Operands swapped (B rows as the MFMA "A" matrix) so that a lane ends up
     // with 4 consecutive n for one m.
-    auto mma = [&](frag(&a)[NB], frag(&b)[NB]) {
+    auto mma = [&](int q) {
 #pragma unroll
         for (int i = 0; i < NB; ++i)
 #pragma unroll
-            for (int j = 0; j < NB; ++j) acc[i][j] = Mma<T>::run(b[j], a[i], acc[i][j]);
+            for (int j = 0; j < NB; ++j) acc[i][j] = Mma<T>::run(fb[q][j], fa[q][i], acc[i][j]);
     };
-    // Scheduling hint for one quarter step of NB*NB MFMAs: the LDS reads of the
-    // next quarter go out one per MFMA at the front, so the remaining MFMAs
-    // cover their latency and the wait at the end of the quarter does not stall;
-    // the HBM->LDS copies follow, one per MFMA.
+    // Scheduling hint for one quarter step of NB*NB MFMAs: LDS reads go out one
+    // per MFMA at the front, so that the MFMAs behind them cover their latency
+    // and the wait at the end of the quarter does not stall; the HBM->LDS copies
+    // follow, one per MFMA.
     auto interleave = [&](auto reads_c, auto copies_c) {
         constexpr int reads = decltype(reads_c)::value;
         constexpr int copies = decltype(copies_c)::value;
@@ -287,72 +289,81 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         }
         __builtin_amdgcn_sched_group_barrier(0x008, NM, 0);  // whatever MFMAs are left
     };
-    template_int<2 * NB> all_reads;
-    template_int<0> none;
+    constexpr int FR = 2 * NB;   // LDS reads per quarter's fragments
     template_int<0> first_half;
     template_int<1> second_half;
-
-    // One quarter step: read the fragments of the next quarter into (an, bn),
-    // optionally issue half a panel of copies, run the MFMAs on (ac, bc).
-    auto quarter = [&](int rbuf, int rko, frag(&an)[NB], frag(&bn)[NB], frag(&ac)[NB], frag(&bc)[NB], auto read_c,
-                       auto copy_c, int ckt, int cbuf, auto half_c) {
-        constexpr bool READ = decltype(read_c)::value;
-        constexpr bool COPY = decltype(copy_c)::value;
-        if constexpr (READ) load_frags(rbuf, rko, an, bn);
-        if constexpr (COPY) issue_half(ckt, cbuf, half_c);
-        mma(ac, bc);
-        constexpr int ncopy = COPY ? HALF : 0;
-        if constexpr (READ) interleave(all_reads, template_int<ncopy>{});
-        else interleave(none, template_int<ncopy>{});
+    auto end_quarter = [&](auto pending_reads_c) {
         __builtin_amdgcn_sched_barrier(0);  // nothing moves across the end of a quarter step
-        wait_lds_reads();
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, decltype(pending_reads_c)::value));
         __builtin_amdgcn_sched_barrier(0);
     };
 
     const int NP = K / kBK;   // panels
-    // One k-step on panel kt (in buffer cur).  C1: panel kt+1 exists and its second
-    // half is still to be copied.  NEXT: panel kt+1 exists.  C2: panel kt+2 exists.
-    auto kstep = [&](int kt, int cur, auto c1_c, auto next_c, auto c2_c) {
+    // One k-step on panel kt (in buffer cur); on entry the fragments of its first
+    // quarter are in registers.  All LDS reads of the panel are issued in the
+    // first two quarters, so the barrier that frees its buffer comes after the
+    // second quarter already and the copies of panel kt+2 have two more quarter
+    // steps to land than if they had to wait for the last fragment read.
+    // NEXT: panel kt+1 exists.  C2: panel kt+2 exists.
+    auto kstep = [&](int kt, int cur, auto next_c, auto c2_c) {
         constexpr bool NEXT = decltype(next_c)::value;
-        quarter(cur, ko[1], a1, b1, a0, b0, std::true_type{}, c1_c, kt + 1, cur ^ 1, second_half);
-        quarter(cur, ko[2], a0, b0, a1, b1, std::true_type{}, std::false_type{}, 0, 0, first_half);
-        quarter(cur, ko[3], a1, b1, a0, b0, std::true_type{}, std::false_type{}, 0, 0, first_half);
+        constexpr bool C2 = decltype(c2_c)::value;
+        // quarter 0: fragments of quarters 1 and 2 go out, only quarter 1's are awaited
+        load_frags(cur, 1);
+        load_frags(cur, 2);
+        mma(0);
+        interleave(template_int<2 * FR>{}, template_int<0>{});
+        end_quarter(template_int<FR>{});
+        // quarter 1: fragments of quarter 3
+        load_frags(cur, 3);
+        mma(1);
+        interleave(template_int<FR>{}, template_int<0>{});
+        end_quarter(template_int<0>{});
         if constexpr (NEXT) {
             // Panel kt+1 has landed for every wave, and every wave has read panel kt
             // for the last time, so its buffer can take panel kt+2.
             wait_vmcnt<0>();
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
-            quarter(cur ^ 1, ko[0], a0, b0, a1, b1, std::true_type{}, c2_c, kt + 2, cur, first_half);
-        } else {
-            quarter(0, 0, a0, b0, a1, b1, std::false_type{}, std::false_type{}, 0, 0, first_half);
         }
+        // quarter 2: first half of panel kt+2
+        if constexpr (C2) issue_half(kt + 2, cur, first_half);
+        mma(2);
+        interleave(template_int<0>{}, template_int<(C2 ? HALF : 0)>{});
+        end_quarter(template_int<0>{});
+        // quarter 3: first fragments of panel kt+1, second half of panel kt+2
+        if constexpr (NEXT) load_frags(cur ^ 1, 0);
+        if constexpr (C2) issue_half(kt + 2, cur, second_half);
+        mma(3);
+        interleave(template_int<(NEXT ? FR : 0)>{}, template_int<(C2 ? HALF : 0)>{});
+        end_quarter(template_int<0>{});
     };
 
-    // Prologue: panel 0 and the first half of panel 1 go out; wait for panel 0.
+    // Prologue: panels 0 and 1 go out; wait for panel 0.
     issue_half(0, 0, first_half);
     issue_half(0, 0, second_half);
     if (NP > 1) {
         issue_half(1, 1, first_half);
-        wait_vmcnt<HALF>();
+        issue_half(1, 1, second_half);
+        wait_vmcnt<LPT>();
     } else {
         wait_vmcnt<0>();
     }
     __builtin_amdgcn_s_barrier();
-    load_frags(0, ko[0], a0, b0);
+    load_frags(0, 0);
     wait_lds_reads();
 
     // The consumer's waves share SIMDs with these waves while a group is being
     // copied; the issue arbiter should always prefer the wave that feeds the MFMAs.
     __builtin_amdgcn_s_setprio(3);
     int kt = 0, cur = 0;
-    for (; kt < NP - 2; ++kt, cur ^= 1) kstep(kt, cur, std::true_type{}, std::true_type{}, std::true_type{});
+    for (; kt < NP - 2; ++kt, cur ^= 1) kstep(kt, cur, std::true_type{}, std::true_type{});
     if (NP >= 2) {
-        kstep(kt, cur, std::true_type{}, std::true_type{}, std::false_type{});
+        kstep(kt, cur, std::true_type{}, std::false_type{});
         ++kt;
         cur ^= 1;
     }
-    kstep(kt, cur, std::false_type{}, std::false_type{}, std::false_type{});
+    kstep(kt, cur, std::false_type{}, std::false_type{});
 
     // ---- epilogue: registers -> LDS strip -> global -------------------------------
     // acc[i][j][4q+r] is element m = 32i + l%32, n = 32j + 8q + 4(l/32) + r.
