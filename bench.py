@@ -29,7 +29,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# BASELINE.json configs; (dtype, M, N, K, tiles per group, world size, eps, a_std, b_std).  A hardware
+# The five benchmark configurations; (dtype, M, N, K, tiles per group, world size, eps, a_std, b_std).  A hardware
 # wave of the GEMM kernel is 256 workgroups x 4 layout tiles = 1024 tiles of 128x128 (W); the tiles of
 # one wave finish together, so groups are whole waves: c3 one wave per group, c4 two ("group size 2").
 # c1 and c2 fit in one wave and keep the tile-count reading of their group sizes (4 and 256 tiles).

@@ -309,7 +309,7 @@ def test_reorder_rmsnorm_undoes_the_permutation():
 
 
 def test_config1_plumbing_run_on_cpu():
-    """BASELINE config 1 end to end on the CPU oracle: fp16 1024^3, 128x128
+    """Benchmark configuration 1 end to end on the CPU oracle: fp16 1024^3, 128x128
     tiles, groups of 4 tiles, reordered output + RMSNorm against fp32."""
     M = N = K = 1024
     BM = BN = 128

@@ -155,7 +155,7 @@ def test_gemm_rejects_unsupported_shapes(L, dev):
 # ---- signalling epilogue -------------------------------------------------------
 
 @pytest.mark.parametrize("dt,M,N,K,algo,w", [
-    (torch.float16, 1024, 1024, 1024, 1, 4),      # BASELINE config 1: 64 tiles, 16 groups of 4 (> TN = 8 counters)
+    (torch.float16, 1024, 1024, 1024, 1, 4),      # benchmark configuration 1: 64 tiles, 16 groups of 4 (> TN = 8 counters)
     (torch.bfloat16, 512, 768, 128, 1, 5),        # ragged last group
     (torch.float16, 1024, 2048, 64, 3, 3),        # 128x256 layout tile
     (torch.bfloat16, 2048, 1024, 64, 5, 7),       # 256x128 layout tile
@@ -384,7 +384,7 @@ def test_reorder_rmsnorm(L, dev, dt, bs, dim, BM, BN, rldn):
     assert O.rel_l2(out.cpu(), ref3) < REL_L2_TOL
 
 
-# ---- BASELINE configurations, full size ------------------------------------------
+# ---- the five benchmark configurations, full size ------------------------------------------
 
 def _full_path(L, dev, comm_stream, dt, M, N, K, w, eps, ws=1, a_std=None, b_std=None, check_rows=None):
     """Whole hot path on random inputs at full size: signalling GEMM overlapped
