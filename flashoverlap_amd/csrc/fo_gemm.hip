@@ -126,15 +126,6 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 template <int N>
 using template_int = std::integral_constant<int, N>;
 
-// f(integral_constant<0>) ... f(integral_constant<N-1>)
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (N > 0) {
-        static_for<N - 1>(f);
-        f(template_int<N - 1>{});
-    }
-}
-
 // STORE: 0 cached, 1 write-through tile stores; REL: 0 release atomic, 1 relaxed atomic.
 template <typename T, int MT, int MODE, int STORE, int REL>
 __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
