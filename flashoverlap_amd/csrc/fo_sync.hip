@@ -50,19 +50,22 @@ __global__ void wait_kernel(int that, int* addr, long long ticks) {
 
 constexpr int kCopyThreads = 512;  // consumer workgroup size
 constexpr int kCopyUnroll = 8;     // 16-byte units in flight per thread
+constexpr long long kUnitsPerTeamMember = 8192;  // 128 KiB: what one workgroup takes of a group before another joins
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// Copies n 16-byte units (n * 16 < 4 GiB); the workgroups of the grid interleave
-// in chunks of kCopyThreads * kCopyUnroll units, every thread keeping kCopyUnroll
-// loads in flight.  COHERENT: read with agent-scope loads that do not hit in
-// the non-coherent caches (for data another XCD wrote while this kernel runs).
+// Copies n 16-byte units (n * 16 < 4 GiB) as member `me` of a team of `team`
+// workgroups, which interleave in chunks of kCopyThreads * kCopyUnroll units,
+// every thread keeping kCopyUnroll loads in flight.  COHERENT: read with
+// agent-scope loads that do not hit in the non-coherent caches (for data
+// another XCD wrote while this kernel runs).
 template <bool COHERENT>
-__device__ __forceinline__ void grid_copy(const uint4* __restrict__ s, uint4* __restrict__ d, long long n) {
+__device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __restrict__ d, long long n, int me,
+                                          int team) {
     const long long chunk = (long long)kCopyThreads * kCopyUnroll;
     [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc;
     if constexpr (COHERENT) rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, 0xffffffff, 0x00020000);
-    for (long long base = (long long)blockIdx.x * chunk; base < n; base += (long long)gridDim.x * chunk) {
+    for (long long base = (long long)me * chunk; base < n; base += (long long)team * chunk) {
         u32x4 v[kCopyUnroll];
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
@@ -81,14 +84,20 @@ __device__ __forceinline__ void grid_copy(const uint4* __restrict__ s, uint4* __
 }
 
 // Persistent form of the host loop in src/overlap_impl.cu:257-265 (and
-// :312-323 for the ReduceScatter receive layout): walks the groups in index
-// order; all workgroups cooperate on each group's copy.  A group's range is
-// cut into nslices equal parts; parts slice_first .. slice_first+slice_count-1
-// are copied, part k to dst + (k - slice_first)*stride + offset/nslices (the
-// receive layout of a ReduceScatter; nslices = 1 is the plain copy).  After its
-// stripe a workgroup bumps MM[g] once more; the workgroup that brings it to
-// cSeg[g] + gridDim.x is the last one out and stores the 0.  It needs few
-// registers and no LDS to speak of, so its waves fit beside a resident GEMM
+// :312-323 for the ReduceScatter receive layout).  Every workgroup walks the
+// groups in index order.  A group is handled by a team of workgroups whose
+// size grows with the group (one member per 128 KiB, at most the whole grid);
+// the teams of consecutive groups are consecutive windows of the grid, so many
+// small groups are spread over the workgroups and one large group is copied by
+// all of them.  A member waits for the group's count, bumps MM[g] once more
+// (the member that brings it to cSeg[g] + team is the last to have seen the
+// count and stores the 0) and copies its stripe of the range.  With the whole grid on every group
+// the groups are released strictly in index order; smaller teams release
+// groups as they complete.  A group's range is cut into nslices equal parts;
+// parts slice_first .. slice_first+slice_count-1 are copied, part k to
+// dst + (k - slice_first)*stride + offset/nslices (the receive layout of a
+// ReduceScatter; nslices = 1 is the plain copy).  The kernel needs few
+// registers and next to no LDS, so its waves fit beside a resident GEMM
 // workgroup on the same CU.
 __global__ void __launch_bounds__(kCopyThreads) wait_consume_kernel(const int* __restrict__ cseg, int G, int* MM,
                                                                     const uint4* __restrict__ src,
@@ -96,37 +105,108 @@ __global__ void __launch_bounds__(kCopyThreads) wait_consume_kernel(const int* _
                                                                     int nslices, int slice_first, int slice_count,
                                                                     long long slice_stride_units, int* order_log,
                                                                     long long ticks) {
-    __shared__ int s_ok;
+    // The groups are taken kCopyThreads at a time: one thread per group works out
+    // where the group starts and which window of the grid is its team (two block
+    // scans), the groups this workgroup belongs to are compacted into a list in
+    // index order, and the list is then worked off.
+    __shared__ int s_ok[2];
+    __shared__ long long s_units[kCopyThreads];
+    __shared__ int s_team[kCopyThreads];
+    __shared__ int s_pos[kCopyThreads];
+    __shared__ long long s_lo[kCopyThreads];
+    __shared__ int s_g[kCopyThreads], s_me[kCopyThreads], s_tm[kCopyThreads];
     const int tid = threadIdx.x;
-    long long lo = 0;  // first 16-byte unit of group g in src
-    for (int g = 0; g < G; ++g) {
-        const int need = cseg[g];
-        if (tid == 0) {
-            const bool ok = bounded_poll(MM + g, ticks, [need](int v) { return v >= need; });
-            if (!ok) atomicAdd(&g_wait_timeouts, 1);
-            s_ok = ok;
+    const int nb = gridDim.x;
+    long long lo_base = 0;  // first 16-byte unit of the chunk's first group
+    int start_base = 0;     // first workgroup of that group's team
+    int mine = 0;           // groups this workgroup has taken part in
+    for (int g0 = 0; g0 < G; g0 += kCopyThreads) {
+        const int g = g0 + tid;
+        long long units = 0;
+        int team = 0;
+        if (g < G) {
+            units = tile_units * cseg[g];
+            const long long want = (units + kUnitsPerTeamMember - 1) / kUnitsPerTeamMember;
+            team = (int)(want < 1 ? 1 : (want > nb ? nb : want));
+        }
+        // inclusive scans of units and team sizes over the chunk
+        s_units[tid] = units;
+        s_team[tid] = team;
+        __syncthreads();
+        for (int off = 1; off < kCopyThreads; off <<= 1) {
+            const long long u = tid >= off ? s_units[tid - off] : 0;
+            const int t = tid >= off ? s_team[tid - off] : 0;
+            __syncthreads();
+            s_units[tid] += u;
+            s_team[tid] += t;
+            __syncthreads();
+        }
+        const long long lo = lo_base + s_units[tid] - units;
+        const int start = (int)(((long long)start_base + s_team[tid] - team) % nb);
+        int me = (int)blockIdx.x - start;   // the team is a window of the grid
+        if (me < 0) me += nb;
+        const int own = (g < G && me < team) ? 1 : 0;
+        // compaction: position of every owned group in the list
+        s_pos[tid] = own;
+        __syncthreads();
+        for (int off = 1; off < kCopyThreads; off <<= 1) {
+            const int c = tid >= off ? s_pos[tid - off] : 0;
+            __syncthreads();
+            s_pos[tid] += c;
+            __syncthreads();
+        }
+        const int count = s_pos[kCopyThreads - 1];
+        const long long chunk_units = s_units[kCopyThreads - 1];
+        const int chunk_team = s_team[kCopyThreads - 1];
+        if (own) {
+            const int at = s_pos[tid] - 1;
+            s_g[at] = g;
+            s_me[at] = me;
+            s_tm[at] = team;
+            s_lo[at] = lo;
         }
         __syncthreads();
-        if (!s_ok) return;  // uniform: the whole workgroup leaves
-        const long long units = tile_units * need;
-        const long long part = units / nslices;
-        for (int k = 0; k < slice_count; ++k)
-            grid_copy<true>(src + lo + (slice_first + k) * part, dst + k * slice_stride_units + lo / nslices, part);
-        __syncthreads();
-        if (tid == 0) {
-            const int old = __hip_atomic_fetch_add(MM + g, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (old == need + (int)gridDim.x - 1)
-                __hip_atomic_store(MM + g, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (order_log && blockIdx.x == 0) order_log[g] = g;
+        for (int i = 0; i < count; ++i) {
+            const int gg = s_g[i], tm = s_tm[i], mem = s_me[i];
+            const long long glo = s_lo[i];
+            const int need = cseg[gg];
+            int* ok_flag = s_ok + (mine++ & 1);   // two flags in turn: lane 0 may already be polling the next group
+            if (tid == 0) {
+                const bool ok = bounded_poll(MM + gg, ticks, [need](int v) { return v >= need; });
+                if (!ok) atomicAdd(&g_wait_timeouts, 1);
+                *ok_flag = ok;
+            }
+            __syncthreads();
+            if (!*ok_flag) return;  // uniform: the whole workgroup leaves
+            if (tid == 0) {
+                // Every member has seen the full count once it has bumped it; the last one
+                // to do so puts the counter back.  The copies need not be finished for that:
+                // the next writer of the counter is ordered behind this kernel.
+                bool last = tm == 1;
+                if (!last)
+                    last = __hip_atomic_fetch_add(MM + gg, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                           need + tm - 1;
+                if (last) {
+                    __hip_atomic_store(MM + gg, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (order_log) order_log[gg] = gg;
+                }
+            }
+            const long long gunits = tile_units * need;
+            const long long part = gunits / nslices;
+            for (int k = 0; k < slice_count; ++k)
+                team_copy<true>(src + glo + (slice_first + k) * part, dst + k * slice_stride_units + glo / nslices,
+                                part, mem, tm);
         }
-        lo += units;
+        __syncthreads();   // the list is rewritten for the next chunk
+        lo_base += chunk_units;
+        start_base = (int)(((long long)start_base + chunk_team) % nb);
     }
 }
 
 __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                                long long units, const unsigned short* src_tail,
                                                                unsigned short* dst_tail, int tail) {
-    grid_copy<false>(src, dst, units);
+    team_copy<false>(src, dst, units, blockIdx.x, gridDim.x);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 

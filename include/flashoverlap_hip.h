@@ -133,9 +133,11 @@ int fo_wait(int that, int* addr, void* stream);
  * src/overlap_impl.cu:257-265); nslices == world size with one slice is what a
  * rank receives from the per-group ReduceScatter (src/overlap_impl.cu:312-323),
  * with all slices it is every rank's receive buffer side by side.
- * order_log (optional, G ints) receives the release sequence.  All nblocks
- * workgroups cooperate on every group, so groups are released strictly in
- * index order. */
+ * Of the nblocks workgroups a team of one per 128 KiB of the group (at most
+ * all) handles a group; consecutive groups go to consecutive teams.  Groups of
+ * nblocks x 128 KiB and more are therefore released strictly in index order by
+ * the whole grid, smaller ones as they complete.  order_log (optional, G ints)
+ * gets order_log[g] = g when group g has been released and its counter reset. */
 int fo_wait_consume(const int* cseg_dev, int G, int* MM,
                     const void* src, void* dst, long long tile_elems,
                     int nslices, int slice_first, int slice_count, long long slice_stride,
