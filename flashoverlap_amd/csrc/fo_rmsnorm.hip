@@ -34,7 +34,7 @@ struct Vec8<__bf16> {
     using type = bf16x8;
 };
 
-constexpr int kRowsPerBlock = 1;  // one wavefront per row, one row per workgroup
+constexpr int kRowsPerBlock = 4;  // one wavefront per row; neighbouring rows read neighbouring tile segments
 
 enum { kNormPlain = 0, kNormGather = 1, kNormGatherFast = 2 };
 
