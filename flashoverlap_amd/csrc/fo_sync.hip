@@ -91,9 +91,10 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
 // small groups are spread over the workgroups and one large group is copied by
 // all of them.  A member waits for the group's count, bumps MM[g] once more
 // (the member that brings it to cSeg[g] + team is the last to have seen the
-// count and stores the 0) and copies its stripe of the range.  With the whole grid on every group
-// the groups are released strictly in index order; smaller teams release
-// groups as they complete.  A group's range is cut into nslices equal parts;
+// count and stores the 0) and copies its stripe of the range.  With the whole
+// grid on every group the groups are released strictly in index order;
+// smaller teams release groups as they complete.  A group's range is cut into
+// nslices equal parts;
 // parts slice_first .. slice_first+slice_count-1 are copied, part k to
 // dst + (k - slice_first)*stride + offset/nslices (the receive layout of a
 // ReduceScatter; nslices = 1 is the plain copy).  The kernel needs few
