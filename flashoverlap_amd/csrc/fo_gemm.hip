@@ -33,6 +33,7 @@
 // with the reference's MUTlass mainloop.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <string_view>
 #include <type_traits>
 
@@ -422,10 +423,14 @@ static int launch_one(const GemmParams& p, hipStream_t stream) {
     constexpr int smem_bytes = 2 * 2 * MT * kRowBytes;
     static_assert(4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the panel buffers");
     auto kern = gemm_kernel<T, MT, MODE, STORE, REL>;
-    static bool configured = false;  // attribute is per function, set once
-    if (!configured) {
+    // The attribute belongs to the function on one device: set it once per device.
+    static std::atomic<unsigned long long> configured{0};
+    int dev = 0;
+    FO_HIP(hipGetDevice(&dev));
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (!(configured.load(std::memory_order_acquire) & bit)) {
         FO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes));
-        configured = true;
+        configured.fetch_or(bit, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, dim3(p.GM * p.GN), dim3(256), smem_bytes, stream, p);
     FO_HIP(hipGetLastError());
