@@ -136,7 +136,9 @@ __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __
                 const T y = (T)((float)xv[k][e] * scale);
                 o[e] = (T)((float)y * (float)gv[k][e]);
             }
-            *(vec*)(orow + (c << 3)) = o;
+            // streaming store: the result is not read again here, and it must not
+            // displace the GEMM operands held in the memory-side cache
+            __builtin_nontemporal_store(o, (vec*)(orow + (c << 3)));
         }
     }
 }
