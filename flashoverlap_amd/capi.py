@@ -26,6 +26,7 @@ SIGNATURES = {
     "fo_gemm": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "fo_gemm_signal": (_i, [_i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "fo_gemm_scatter": (_i, [_i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
+    "fo_gemm_signal_static": (_i, [_i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "fo_build_group_table": (_i, [_vp, _i, _i, _vp, _vp]),
     "fo_raster_hint": (_i, [_i, _i, _i, _ip]),
     "fo_tune": (_i, [C.c_char_p, _i]),

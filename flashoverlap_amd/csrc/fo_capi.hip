@@ -84,6 +84,11 @@ int fo_gemm_scatter(int dtype, int algo, int M, int N, int K, int rLDN, const in
                        (hipStream_t)stream);
 }
 
+int fo_gemm_signal_static(int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg_dev, int G,
+                          const void* A, const void* B, void* D, int* MM, const int* RA, int monitor, void* stream) {
+    return gemm_signal_static(dtype, algo, M, N, K, rLDN, cseg_dev, G, A, B, D, MM, RA, monitor, (hipStream_t)stream);
+}
+
 int fo_build_group_table(const int* cseg_dev, int G, int T, int* group_table, void* stream) {
     return launch_group_table(cseg_dev, G, T, group_table, (hipStream_t)stream);
 }

@@ -29,6 +29,10 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
 int raster_hint(int algo, int M, int N, int* hint);
 int tune(const char* key, int value);
 
+// fo_static.hip
+int gemm_signal_static(int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg, int G, const void* A,
+                       const void* B, void* D, int* MM, const int* RA, int monitor, hipStream_t stream);
+
 // fo_sync.hip
 int launch_group_table(const int* cseg, int G, int T, int* table, hipStream_t stream);
 int launch_wait(int that, int* addr, hipStream_t stream);

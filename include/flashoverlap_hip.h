@@ -92,6 +92,24 @@ int fo_gemm_scatter(int dtype, int algo, int M, int N, int K, int rLDN,
                     const void* A, const void* B, void* D,
                     int* MM, const int* RA, const int* RE, int monitor, void* stream);
 
+/* fo_gemm_signal for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  The slot->group table, which
+ * fo_gemm_signal takes from its caller as `group_table`, is built by this call
+ * (on `stream`, ahead of the GEMM) in a device array that is part of the
+ * library image: FO_STATIC_MAX_TILES ints (256 KiB) per GPU, held until the
+ * process ends.  The call allocates and frees nothing.  Shapes with more than
+ * FO_STATIC_MAX_TILES layout tiles are rejected with FO_ERR_LIMIT.  All calls
+ * on one GPU share that GPU's array: calls whose kernels may run concurrently
+ * on one GPU (different streams) race on it; calls ordered on one stream, or
+ * otherwise serialised, are safe and need no clearing in between.  Results are
+ * identical to fo_gemm_signal with a table from fo_build_group_table. */
+#define FO_STATIC_MAX_TILES 65536
+int fo_gemm_signal_static(int dtype, int algo, int M, int N, int K, int rLDN,
+                          const int* cseg_dev, int G,
+                          const void* A, const void* B, void* D,
+                          int* MM, const int* RA, int monitor, void* stream);
+
 /* group_table[s] = group(s) for s in [0,T), computed on the device from
  * cseg_dev.  No counterpart in the reference, whose epilogue rescans cSeg for
  * every tile (src/overlap/gemm_with_signal.h:188-193); results are identical. */
