@@ -6,18 +6,24 @@
 // (MT/64)^2 blocks of v_mfma_f32_32x32x16, accumulators in AGPRs.
 //
 // Main loop: A and B panels of 64 k-elements stream HBM -> LDS with
-// buffer_load_dwordx4 ... lds (no register staging) into two LDS buffers.  A
-// panel row is 128 bytes, so every copy instruction fetches eight whole cache
-// lines: the L2 serves one request per channel per clock whatever its size, and
-// at this tile size the kernel sits at the edge of that request rate, so
-// half-line requests cost a quarter of the throughput.  The 16-byte chunks of a
-// row are XOR-swizzled by row so the ds_read_b128 fragment reads are
-// bank-conflict free.  A k-step of 64 is four quarter steps of 16 MFMAs each;
-// the fragments of all four are read during the first two, so while one
-// quarter's MFMAs run the fragments of the next are already in registers, and
-// the workgroup barrier that hands the panel's buffer to the copies of panel
-// p+2 sits in the middle of the k-step, two quarter steps before the last MFMA
-// on that panel.  There is one barrier per k-step.
+// buffer_load_dwordx4 ... lds (no register staging) into a ring of five panel
+// slots (all of the 160 KiB of LDS at MT = 256): the A and B panels of the
+// k-step being multiplied, those of the next one, and one free slot.  A panel
+// row is 128 bytes, so every copy instruction fetches eight whole cache lines:
+// the L2 serves one request per channel per clock whatever its size, and at
+// this tile size the kernel sits at the edge of that request rate, so half-line
+// requests cost a quarter of the throughput.  The 16-byte chunks of a row are
+// XOR-swizzled by row so the ds_read_b128 fragment reads are bank-conflict
+// free.  A k-step of 64 is four quarter steps of 16 MFMAs each; the fragments
+// of all four are read during the first two, so while one quarter's MFMAs run
+// the fragments of the next are already in registers, and the workgroup
+// barrier that releases the panel's two slots sits in the middle of the
+// k-step.  The free slot lets the copies of A(p+2) go out in the first half of
+// k-step p and those of B(p+2) in the second half: the same number of copies
+// in every quarter step, and between one and three more quarter steps for
+// them to land than with two buffers, which is what the kernel needs when its
+// operands come from HBM and not from the memory-side cache.  There is one
+// barrier per k-step.
 //
 // Epilogue: the quadrant goes through LDS in strips of 32 rows so that every
 // global store instruction writes four whole 256-byte row segments, either to
@@ -132,8 +138,7 @@ template <typename T, int MT, int MODE, int STORE, int REL>
 __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     constexpr int WT = MT / 2;               // wave quadrant edge
     constexpr int NB = WT / 32;              // 32x32 MFMA blocks per quadrant edge
-    constexpr int PANEL = MT * kRowBytes;    // bytes of one A (or B) panel
-    constexpr int BUF = 2 * PANEL;           // one LDS buffer: A panel, then B panel
+    constexpr int PANEL = MT * kRowBytes;    // bytes of one A (or B) panel = one LDS slot
     constexpr int LOADS = MT / 32;           // wave-wide 1 KiB copies per wave per panel
     constexpr int LPT = 2 * LOADS;           // copies per wave per k-step
     constexpr int HALF = LPT / 2;
@@ -204,28 +209,33 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     const unsigned slab_bytes = 8u * (unsigned)K * 2u;    // bytes between consecutive slabs
     const int lds_cp = wave * (LOADS * 1024);             // this wave's first slab in a panel
 
-    // Buffer `buf` receives panel `kt`; the copies of a panel are issued in two
-    // halves so that they can be spread over two quarter steps.
-    auto issue_half = [&](int kt, int buf, auto half_c) {
+    // The LDS is a ring of five panel slots.  Panel units alternate A(0) B(0)
+    // A(1) B(1) ...; unit u lives in slot u % 5.  `slot` is the byte offset of
+    // the receiving slot; the copies of a unit are issued in two halves.
+    auto issue_unit = [&](int kt, int slot, auto isb_c, auto half_c) {
+        constexpr bool ISB = decltype(isb_c)::value;
         constexpr int H = decltype(half_c)::value;
-        unsigned char* sA = smem + buf * BUF + lds_cp;
-        unsigned char* sB = sA + PANEL;
+        unsigned char* dst = smem + slot + lds_cp;
         const unsigned koff = (unsigned)kt * (kBK * 2);
 #pragma unroll
         for (int j = H * (LOADS / 2); j < (H + 1) * (LOADS / 2); ++j) {
             const int voff = (j & 1) ? cp_off1 : cp_off0;   // LOADS*8 is a multiple of 16: slab parity = j parity
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(sA + j * 1024), 16, voff,
-                                                     (int)(baseA + j * slab_bytes + koff), 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(sB + j * 1024), 16, voff,
-                                                     (int)(baseB + j * slab_bytes + koff), 0, 0);
+            if constexpr (ISB)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, voff,
+                                                         (int)(baseB + j * slab_bytes + koff), 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(dst + j * 1024), 16, voff,
+                                                         (int)(baseA + j * slab_bytes + koff), 0, 0);
         }
     };
+    std::false_type unit_a;
+    std::true_type unit_b;
 
     // ---- LDS -> register fragment addressing ----------------------------------
     // MFMA 32x32x16 operand: lane l supplies row l%32, k = 8*(l/32) .. +7.
     const int fr_row = lane & 31, fr_h = lane >> 5;
     const int a_lane = (wm * WT + fr_row) * kRowBytes;
-    const int b_lane = PANEL + (wn * WT + fr_row) * kRowBytes;
+    const int b_lane = (wn * WT + fr_row) * kRowBytes;
     int ko[4];   // chunk offset of each quarter step (k 0..15, 16..31, 32..47, 48..63)
 #pragma unroll
     for (int q = 0; q < 4; ++q) ko[q] = ((2 * q + fr_h) ^ swz(fr_row)) * 16;
@@ -241,12 +251,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     // Fragments of the four quarter steps of a panel (k 0..15, 16..31, 32..47, 48..63).
     frag fa[4][NB], fb[4][NB];
 
-    auto load_frags = [&](int buf, int q) {
-        const unsigned char* base = smem + buf * BUF + ko[q];
+    auto load_frags = [&](int slot_a, int slot_b, int q) {
+        const unsigned char* pa = smem + slot_a + ko[q] + a_lane;
+        const unsigned char* pb = smem + slot_b + ko[q] + b_lane;
 #pragma unroll
-        for (int i = 0; i < NB; ++i) fa[q][i] = *(const frag*)(base + a_lane + i * BLK);
+        for (int i = 0; i < NB; ++i) fa[q][i] = *(const frag*)(pa + i * BLK);
 #pragma unroll
-        for (int j = 0; j < NB; ++j) fb[q][j] = *(const frag*)(base + b_lane + j * BLK);
+        for (int j = 0; j < NB; ++j) fb[q][j] = *(const frag*)(pb + j * BLK);
     };
     // Operands swapped (B rows as the MFMA "A" matrix) so that a lane ends up
     // with 4 consecutive n for one m.
@@ -291,71 +302,89 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     };
 
     const int NP = K / kBK;   // panels
-    // One k-step on panel kt (in buffer cur); on entry the fragments of its first
-    // quarter are in registers.  All LDS reads of the panel are issued in the
-    // first two quarters, so the barrier that frees its buffer comes after the
-    // second quarter already and the copies of panel kt+2 have two more quarter
-    // steps to land than if they had to wait for the last fragment read.
+    // One k-step on panel kt, whose A and B units sit in slots sa and sb; the
+    // units of panel kt+1 are in na and nb (landed or landing), sp is the free
+    // slot.  On entry the fragments of the first quarter are in registers.  All
+    // LDS reads of the panel are issued in the first two quarters, so sa and sb
+    // are handed over at the barrier in the middle of the k-step.  A(kt+2) goes
+    // to the free slot during the first half of the k-step, B(kt+2) to slot sa
+    // during the second half.
     // NEXT: panel kt+1 exists.  C2: panel kt+2 exists.
-    auto kstep = [&](int kt, int cur, auto next_c, auto c2_c) {
+    constexpr int QC = LOADS / 2;   // copies per quarter per wave
+    auto kstep = [&](int kt, int sa, int sb, int na, int nb, int sp, auto next_c, auto c2_c) {
         constexpr bool NEXT = decltype(next_c)::value;
         constexpr bool C2 = decltype(c2_c)::value;
         // quarter 0: fragments of quarters 1 and 2 go out, only quarter 1's are awaited
-        load_frags(cur, 1);
-        load_frags(cur, 2);
+        load_frags(sa, sb, 1);
+        load_frags(sa, sb, 2);
+        if constexpr (C2) issue_unit(kt + 2, sp, unit_a, first_half);
         mma(0);
-        interleave(template_int<2 * FR>{}, template_int<0>{});
+        interleave(template_int<2 * FR>{}, template_int<(C2 ? QC : 0)>{});
         end_quarter(template_int<FR>{});
         // quarter 1: fragments of quarter 3
-        load_frags(cur, 3);
+        load_frags(sa, sb, 3);
+        if constexpr (C2) issue_unit(kt + 2, sp, unit_a, second_half);
         mma(1);
-        interleave(template_int<FR>{}, template_int<0>{});
+        interleave(template_int<FR>{}, template_int<(C2 ? QC : 0)>{});
         end_quarter(template_int<0>{});
         if constexpr (NEXT) {
-            // Panel kt+1 has landed for every wave, and every wave has read panel kt
-            // for the last time, so its buffer can take panel kt+2.
-            wait_vmcnt<0>();
+            // Panel kt+1 has landed for every wave (the copies of A(kt+2), the newest
+            // LOADS of this wave, may still be in flight: copies complete in issue
+            // order), and every wave has read panel kt for the last time.
+            if constexpr (C2) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
         }
-        // quarter 2: first half of panel kt+2
-        if constexpr (C2) issue_half(kt + 2, cur, first_half);
+        // quarter 2: first half of B(kt+2) into the slot A(kt) just left
+        if constexpr (C2) issue_unit(kt + 2, sa, unit_b, first_half);
         mma(2);
-        interleave(template_int<0>{}, template_int<(C2 ? HALF : 0)>{});
+        interleave(template_int<0>{}, template_int<(C2 ? QC : 0)>{});
         end_quarter(template_int<0>{});
-        // quarter 3: first fragments of panel kt+1, second half of panel kt+2
-        if constexpr (NEXT) load_frags(cur ^ 1, 0);
-        if constexpr (C2) issue_half(kt + 2, cur, second_half);
+        // quarter 3: first fragments of panel kt+1, second half of B(kt+2)
+        if constexpr (NEXT) load_frags(na, nb, 0);
+        if constexpr (C2) issue_unit(kt + 2, sa, unit_b, second_half);
         mma(3);
-        interleave(template_int<(NEXT ? FR : 0)>{}, template_int<(C2 ? HALF : 0)>{});
+        interleave(template_int<(NEXT ? FR : 0)>{}, template_int<(C2 ? QC : 0)>{});
         end_quarter(template_int<0>{});
     };
 
     // Prologue: panels 0 and 1 go out; wait for panel 0.
-    issue_half(0, 0, first_half);
-    issue_half(0, 0, second_half);
+    issue_unit(0, 0 * PANEL, unit_a, first_half);
+    issue_unit(0, 0 * PANEL, unit_a, second_half);
+    issue_unit(0, 1 * PANEL, unit_b, first_half);
+    issue_unit(0, 1 * PANEL, unit_b, second_half);
     if (NP > 1) {
-        issue_half(1, 1, first_half);
-        issue_half(1, 1, second_half);
+        issue_unit(1, 2 * PANEL, unit_a, first_half);
+        issue_unit(1, 2 * PANEL, unit_a, second_half);
+        issue_unit(1, 3 * PANEL, unit_b, first_half);
+        issue_unit(1, 3 * PANEL, unit_b, second_half);
         wait_vmcnt<LPT>();
     } else {
         wait_vmcnt<0>();
     }
     __builtin_amdgcn_s_barrier();
-    load_frags(0, 0);
+    load_frags(0, PANEL, 0);
     wait_lds_reads();
 
     // The consumer's waves share SIMDs with these waves while a group is being
     // copied; the issue arbiter should always prefer the wave that feeds the MFMAs.
     __builtin_amdgcn_s_setprio(3);
-    int kt = 0, cur = 0;
-    for (; kt < NP - 2; ++kt, cur ^= 1) kstep(kt, cur, std::true_type{}, std::true_type{});
-    if (NP >= 2) {
-        kstep(kt, cur, std::true_type{}, std::false_type{});
-        ++kt;
-        cur ^= 1;
+    int kt = 0;
+    int sa = 0, sb = PANEL, na = 2 * PANEL, nb = 3 * PANEL, sp = 4 * PANEL;
+    auto rotate = [&]() {   // (sa, sb, na, nb, sp) <- (na, nb, sp, sa, sb)
+        const int a0 = sa, b0 = sb;
+        sa = na; sb = nb; na = sp; nb = a0; sp = b0;
+    };
+    for (; kt < NP - 2; ++kt) {
+        kstep(kt, sa, sb, na, nb, sp, std::true_type{}, std::true_type{});
+        rotate();
     }
-    kstep(kt, cur, std::false_type{}, std::false_type{});
+    if (NP >= 2) {
+        kstep(kt, sa, sb, na, nb, sp, std::true_type{}, std::false_type{});
+        rotate();
+        ++kt;
+    }
+    kstep(kt, sa, sb, na, nb, sp, std::false_type{}, std::false_type{});
 
     // ---- epilogue: registers -> LDS strip -> global -------------------------------
     // acc[i][j][4q+r] is element m = 32i + l%32, n = 32j + 8q + 4(l/32) + r.
@@ -420,8 +449,8 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 
 template <typename T, int MT, int MODE, int STORE, int REL>
 static int launch_one(const GemmParams& p, hipStream_t stream) {
-    constexpr int smem_bytes = 2 * 2 * MT * kRowBytes;
-    static_assert(4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the panel buffers");
+    constexpr int smem_bytes = 5 * MT * kRowBytes;   // five panel slots: 160 KiB at MT = 256
+    static_assert(4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the panel slots");
     auto kern = gemm_kernel<T, MT, MODE, STORE, REL>;
     // The attribute belongs to the function on one device: set it once per device.
     static std::atomic<unsigned long long> configured{0};
