@@ -11,11 +11,14 @@ Prints ONE JSON line.  `value` is 2*M*N*K divided by the whole step time.  The
 roofline object is for the dominant kernel (the signalling GEMM) as it ran
 inside the timed steps, from HIP events around every launch on its own stream.
 The same run also times, back to back and on their own, the signalling GEMM
-and its plain twin (signal overhead), reorder+RMSNorm (HBM roofline) and the
-consumer copy, the serial (non-overlapped) step, and a CPU baseline (the
-oracle's fp32 matmul + RMSNorm on the host cores) on a bounded sample of the
-same workload.  Launch order: W+K serial steps, W+K overlapped steps, then the
-isolated kernels (5 warm-up + --kernel-iters + 10 launches each).
+and its plain twin (signal overhead), reorder+RMSNorm (HBM roofline; over a
+rotation of buffer pairs larger than the 256 MB memory-side cache, and inside
+the timed steps) and the consumer copy, the serial (non-overlapped) step, the
+plain GEMM on all-zero operands (what the same instruction stream does when
+the chip is not power-limited), and a CPU baseline (the oracle's fp32 matmul +
+RMSNorm on the host cores) on a bounded sample of the same workload.  Launch
+order: W+K serial steps, W+K overlapped steps, then the isolated kernels
+(5 warm-up + --kernel-iters + 10 launches each).
 """
 from __future__ import annotations
 
@@ -31,16 +34,20 @@ sys.path.insert(0, ROOT)
 
 # The five benchmark configurations; (dtype, M, N, K, tiles per group, world size, eps, a_std, b_std).  A hardware
 # wave of the GEMM kernel is 256 workgroups x 4 layout tiles = 1024 tiles of 128x128 (W); the tiles of
-# one wave finish together, so groups are whole waves: c3 one wave per group, c4 two ("group size 2").
-# c1 and c2 fit in one wave and keep the tile-count reading of their group sizes (4 and 256 tiles).
+# one wave finish together.  A "group size g" can be read as g tiles or as g waves (the reference's
+# cSeg counts waves, tune/search.py:502-513).  c3 and c5: one wave per group.  c2 (sweep {1,2,4,8,16}) and
+# c4 (size 2) default to the tile-count reading, which stresses the counters (c4: 4096 groups of 2
+# tiles); `--reading waves` takes the other one (c4: 4 groups of 2048 tiles, c2: one group), and
+# `--group-tiles` sets any size.  `--both-readings` puts the other reading's figures into the same record.
 TILES_PER_WAVE = 1024
 WORKLOADS = {
     "c1": ("fp16", 1024, 1024, 1024, 4, 1, 1e-6, None, None),
-    "c2": ("fp16", 4096, 4096, 4096, 256, 1, 1e-5, None, None),
+    "c2": ("fp16", 4096, 4096, 4096, 4, 1, 1e-5, None, None),
     "c3": ("bf16", 8192, 4096, 7168, TILES_PER_WAVE, 1, 1e-5, 1.0, 0.02),
-    "c4": ("bf16", 16384, 8192, 1024, 2 * TILES_PER_WAVE, 1, 1e-5, None, None),
+    "c4": ("bf16", 16384, 8192, 1024, 2, 1, 1e-5, None, None),
     "c5": ("bf16", 8192, 8192, 3584, TILES_PER_WAVE, 8, 1e-5, None, None),
 }
+WAVE_READING = {"c2": TILES_PER_WAVE, "c4": 2 * TILES_PER_WAVE}   # tiles per group under the wave-count reading
 NAMES = {
     "c1": "fp16 1024^3 plumbing shape",
     "c2": "fp16 4096^3 square GEMM",
@@ -50,11 +57,36 @@ NAMES = {
 }
 PEAK_MFMA_TFLOPS = 2516.6   # MI355X dense fp16/bf16: 256 CU x 4096 FLOP/clk x 2.4 GHz
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+MALL_BYTES = 256 << 20      # memory-side cache: a buffer rotation has to exceed it to measure HBM
 # Bytes that cross the L2 -> memory interface per signalling-GEMM launch, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs of `bench.py --no-overlap` (profiles/gemm_signal_c3_counters.txt):
-# FETCH_SIZE 344245 KiB x 1.999 (the 64 MiB consumer copy reads as 32786.5 KiB) + WRITE_SIZE 65600 KiB
-# x 1.000.  None for workloads that have not been measured.
+# FETCH_SIZE KiB x 1.999 (the 64 MiB consumer copy reads as 32786.5 KiB) + WRITE_SIZE KiB x 1.000.
+# None for workloads that have not been measured.
 MEASURED_TRAFFIC_BYTES = {"c3": 771_800_000}
+
+
+class Timer:
+    """HIP-event timing through the C ABI, on the stream the kernels are launched on."""
+
+    def __init__(self, L, capi, stream=None):
+        self.L, self.capi, self.stream = L, capi, stream
+
+    def event(self):
+        e = C.c_void_p()
+        self.capi.check(self.L.fo_event_create(C.byref(e)))
+        return e
+
+    def record(self, e):
+        self.capi.check(self.L.fo_event_record(e, self.stream))
+
+    def ms(self, e0, e1):
+        v = C.c_float()
+        self.capi.check(self.L.fo_event_elapsed_ms(e0, e1, C.byref(v)))
+        return v.value
+
+    def free(self, *evs):
+        for e in evs:
+            self.capi.check(self.L.fo_event_destroy(e))
 
 
 def main() -> int:
@@ -64,9 +96,14 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--group-tiles", type=int, default=0, help="tiles per signal group (0 = workload default)")
+    ap.add_argument("--reading", default="default", choices=["default", "tiles", "waves"],
+                    help="how a workload's group size is read (c2, c4): as tiles or as hardware waves")
+    ap.add_argument("--both-readings", action="store_true",
+                    help="c2/c4: also time the step under the other reading and put it into the record")
     ap.add_argument("--kernel-iters", type=int, default=100, help="timed launches per isolated kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline work; 0 skips it")
-    ap.add_argument("--consumer-blocks", type=int, default=64, help="workgroups of the persistent consumer")
+    ap.add_argument("--consumer-blocks", type=int, default=0,
+                    help="workgroups of the persistent consumer (0 = one per CU, which is also the maximum)")
     ap.add_argument("--consumer", default="auto", choices=["auto", "per_group", "persistent"])
     ap.add_argument("--no-overlap", action="store_true",
                     help="order the consumer behind the GEMM in the timed step (needed under counter collection, "
@@ -86,8 +123,14 @@ def main() -> int:
     L = capi.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    cu, khz, xcd = C.c_int(), C.c_int(), C.c_int()
+    capi.check(L.fo_device_info(C.byref(cu), C.byref(khz), C.byref(xcd)))
+    if a.consumer_blocks <= 0:
+        a.consumer_blocks = cu.value
 
-    dts, M, N, K, w, ws, eps, a_std, b_std = WORKLOADS[a.workload]
+    dts, M, N, K, w_default, ws, eps, a_std, b_std = WORKLOADS[a.workload]
+    w_tiles, w_waves = w_default, WAVE_READING.get(a.workload, w_default)
+    w = w_waves if a.reading == "waves" else w_tiles
     if a.group_tiles:
         w = a.group_tiles
     dt = torch.float16 if dts == "fp16" else torch.bfloat16
@@ -96,8 +139,6 @@ def main() -> int:
     BM, BN, _ = capi.algo_tile(algo)
     TM, TN = M // BM, N // BN
     T = TM * TN
-    cseg = tiling.uniform_cseg(T, w)
-    G = len(cseg)
 
     # synthetic inputs: generated on the CPU with a fixed seed, cast, uploaded
     torch.manual_seed(0)
@@ -109,45 +150,60 @@ def main() -> int:
     A, B, gamma = A_h.to(dev), B_h.to(dev), g_h.to(dev)
     Cp = torch.empty(M * N, dtype=dt, device=dev)
     Cn = torch.empty(M, N, dtype=dt, device=dev)
-    staging = torch.zeros(M * N, dtype=dt, device=dev)
-    out = torch.empty(M, N, dtype=dt, device=dev)
+    # reorder+RMSNorm reads `staging` and writes `out`; enough pairs that one pass over all of them
+    # exceeds the memory-side cache, so a back-to-back rotation measures HBM and not that cache
+    pair_bytes = 2 * M * N * 2
+    npairs = max(1, -(-MALL_BYTES // pair_bytes) + 1)
+    stagings = [torch.zeros(M * N, dtype=dt, device=dev) for _ in range(npairs)]
+    outs = [torch.empty(M, N, dtype=dt, device=dev) for _ in range(npairs)]
+    staging, out = stagings[0], outs[0]
     hint = tiling.raster_hint(M, N, algo)
     RA = tiling.reorder_indices(T, hint, dev).reshape(TM, TN)
-    RE = tiling.generate_row_remap_array(M, N, BM, BN, cseg, ws, dev) if ws > 1 else None
-    cseg_d = torch.tensor(cseg, dtype=torch.int32, device=dev)
-    MM = torch.zeros(max(G, TN), dtype=torch.int32, device=dev)
-    table = torch.empty(T, dtype=torch.int32, device=dev)
-    capi.check(L.fo_build_group_table(cseg_d.data_ptr(), G, T, table.data_ptr(), None))
     comm = C.c_void_p()
     capi.check(L.fo_stream_create(C.byref(comm)))
     capi.check(L.fo_set_wait_timeout_ms(10000))
     main_stream = None  # the null stream; all launches of the main leg go there
+    tm = Timer(L, capi, main_stream)
 
-    def gemm_signal():
+    class Grouping:
+        """Everything that depends on the group size: cSeg, counters, table, row remap."""
+
+        def __init__(self, w):
+            self.w = w
+            self.cseg = tiling.uniform_cseg(T, w)
+            self.G = len(self.cseg)
+            self.cseg_d = torch.tensor(self.cseg, dtype=torch.int32, device=dev)
+            self.MM = torch.zeros(max(self.G, TN), dtype=torch.int32, device=dev)
+            self.table = torch.empty(T, dtype=torch.int32, device=dev)
+            capi.check(L.fo_build_group_table(self.cseg_d.data_ptr(), self.G, T, self.table.data_ptr(), None))
+            self.RE = tiling.generate_row_remap_array(M, N, BM, BN, self.cseg, ws, dev) if ws > 1 else None
+            # Same rule as OverlapImpl: up to 32 groups the reference's structure (one wait kernel and one
+            # consumer launch per group, src/overlap_impl.cu:257-265), beyond that one persistent kernel.
+            self.per_group = a.consumer == "per_group" or (a.consumer == "auto" and self.G <= 32)
+
+    def gemm_signal(g):
         if ws > 1:
-            capi.check(L.fo_gemm_scatter(code, algo, M, N, K, 1, cseg_d.data_ptr(), G, table.data_ptr(), A.data_ptr(),
-                                         B.data_ptr(), Cp.data_ptr(), MM.data_ptr(), RA.data_ptr(), RE.data_ptr(), 0,
-                                         main_stream))
+            capi.check(L.fo_gemm_scatter(code, algo, M, N, K, 1, g.cseg_d.data_ptr(), g.G, g.table.data_ptr(),
+                                         A.data_ptr(), B.data_ptr(), Cp.data_ptr(), g.MM.data_ptr(), RA.data_ptr(),
+                                         g.RE.data_ptr(), 0, main_stream))
         else:
-            capi.check(L.fo_gemm_signal(code, algo, M, N, K, 1, cseg_d.data_ptr(), G, table.data_ptr(), A.data_ptr(),
-                                        B.data_ptr(), Cp.data_ptr(), MM.data_ptr(), RA.data_ptr(), 0, main_stream))
+            capi.check(L.fo_gemm_signal(code, algo, M, N, K, 1, g.cseg_d.data_ptr(), g.G, g.table.data_ptr(),
+                                        A.data_ptr(), B.data_ptr(), Cp.data_ptr(), g.MM.data_ptr(), RA.data_ptr(), 0,
+                                        main_stream))
 
-    def gemm_plain():
-        capi.check(L.fo_gemm(code, algo, M, N, K, A.data_ptr(), B.data_ptr(), Cn.data_ptr(), main_stream))
+    def gemm_plain(a_t=None, b_t=None):
+        a_t, b_t = (A, B) if a_t is None else (a_t, b_t)
+        capi.check(L.fo_gemm(code, algo, M, N, K, a_t.data_ptr(), b_t.data_ptr(), Cn.data_ptr(), main_stream))
 
-    # Same rule as OverlapImpl: up to 32 groups the reference's structure (one wait kernel and one
-    # consumer launch per group, src/overlap_impl.cu:257-265), beyond that one persistent kernel.
-    per_group = a.consumer == "per_group" or (a.consumer == "auto" and G <= 32)
-
-    def wait_consume():
-        if not per_group:
-            capi.check(L.fo_wait_consume(cseg_d.data_ptr(), G, MM.data_ptr(), Cp.data_ptr(), staging.data_ptr(),
-                                         BM * BN, ws, 0, ws, (M * N // ws) if ws > 1 else 0, None,
-                                         a.consumer_blocks, comm))
+    def wait_consume(g):
+        if not g.per_group:
+            capi.check(L.fo_wait_consume(g.cseg_d.data_ptr(), g.G, g.MM.data_ptr(), Cp.data_ptr(),
+                                         staging.data_ptr(), BM * BN, ws, 0, ws, (M * N // ws) if ws > 1 else 0,
+                                         None, a.consumer_blocks, comm))
             return
         acc = 0
-        for g, n in enumerate(cseg):
-            capi.check(L.fo_wait(n, MM.data_ptr() + 4 * g, comm))
+        for gi, n in enumerate(g.cseg):
+            capi.check(L.fo_wait(n, g.MM.data_ptr() + 4 * gi, comm))
             elems = n * BM * BN
             part = elems // ws
             for k in range(ws):  # ws > 1: slice k of the group goes to rank k's receive buffer
@@ -155,109 +211,129 @@ def main() -> int:
                                         staging.data_ptr() + 2 * (k * (M * N // ws) + acc // ws), 2 * part, comm))
             acc += elems
 
-    def norm():
+    def norm(i=0):
+        x, o = stagings[i], outs[i]
         if ws > 1:  # every rank slice is a layout with tile height BM/ws: ws problems, one launch
-            capi.check(L.fo_reorder_rmsnorm_batched(code, staging.data_ptr(), gamma.data_ptr(), out.data_ptr(), ws,
+            capi.check(L.fo_reorder_rmsnorm_batched(code, x.data_ptr(), gamma.data_ptr(), o.data_ptr(), ws,
                                                     M // ws, N, BM // ws, BN, 1, RA.data_ptr(), eps, main_stream))
         else:
-            capi.check(L.fo_reorder_rmsnorm(code, staging.data_ptr(), gamma.data_ptr(), out.data_ptr(), M, N, BM, BN,
+            capi.check(L.fo_reorder_rmsnorm(code, x.data_ptr(), gamma.data_ptr(), o.data_ptr(), M, N, BM, BN,
                                             1, RA.data_ptr(), eps, main_stream))
 
-    def step(overlap=True, ev=None):
+    def step(g, overlap=True, ev=None):
         if ev:
-            capi.check(L.fo_event_record(ev[0], main_stream))
-        gemm_signal()
+            tm.record(ev[0])
+        gemm_signal(g)
         if ev:
-            capi.check(L.fo_event_record(ev[1], main_stream))
+            tm.record(ev[1])
         if not overlap:  # consumer ordered behind the GEMM: the serial reference for the overlap
             capi.check(L.fo_stream_join(main_stream, comm))
-        wait_consume()
+        wait_consume(g)
         capi.check(L.fo_stream_join(comm, main_stream))
+        if ev:
+            tm.record(ev[2])   # fires once the last group has been consumed
         norm()
+        if ev:
+            tm.record(ev[3])
 
-    def time_steps(overlap):
-        """Wall time per step, and the signalling GEMM's own duration inside those same
-        steps (one HIP event pair per step on the GEMM's stream)."""
-        evs = []
-        for _ in range(a.steps):
-            e0, e1 = C.c_void_p(), C.c_void_p()
-            capi.check(L.fo_event_create(C.byref(e0)))
-            capi.check(L.fo_event_create(C.byref(e1)))
-            evs.append((e0, e1))
+    def time_steps(g, overlap):
+        """Wall time per step, and the durations of the signalling GEMM and of reorder+RMSNorm inside
+        those same steps (HIP events on the stream they run on)."""
+        evs = [tuple(tm.event() for _ in range(4)) for _ in range(a.steps)]
         for _ in range(a.warmup):
-            step(overlap)
+            step(g, overlap)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for ev in evs:
-            step(overlap, ev)
+            step(g, overlap, ev)
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e3 / a.steps
-        v, tot = C.c_float(), 0.0
-        for e0, e1 in evs:
-            capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(v)))
-            tot += v.value
-            capi.check(L.fo_event_destroy(e0))
-            capi.check(L.fo_event_destroy(e1))
-        return wall, tot / a.steps
+        gemm_ms = sum(tm.ms(e[0], e[1]) for e in evs) / a.steps
+        norm_ms = sum(tm.ms(e[2], e[3]) for e in evs) / a.steps
+        for e in evs:
+            tm.free(*e)
+        return wall, gemm_ms, norm_ms
+
+    def check_timeouts():
+        n = C.c_int()
+        capi.check(L.fo_wait_timeouts(C.byref(n), 1))
+        if n.value:
+            print(f"bench.py: {n.value} bounded waits expired; results invalid", file=sys.stderr)
+        return n.value
+
+    def consumer_name(g):
+        return ("one wait kernel + one copy launch per group" if g.per_group else
+                f"persistent wait+consume, {a.consumer_blocks} workgroups")
 
     # ---- whole path: W warm-up steps, then exactly K timed steps -----------------
-    serial_ms, serial_gemm_ms = time_steps(False)
-    step_ms, step_gemm_ms = (serial_ms, serial_gemm_ms) if a.no_overlap else time_steps(True)
-    timeouts = C.c_int()
-    capi.check(L.fo_wait_timeouts(C.byref(timeouts), 1))
-    if timeouts.value:
-        print(f"bench.py: {timeouts.value} bounded waits expired; results invalid", file=sys.stderr)
+    grp = Grouping(w)
+    serial_ms, serial_gemm_ms, serial_norm_ms = time_steps(grp, False)
+    step_ms, step_gemm_ms, step_norm_ms = ((serial_ms, serial_gemm_ms, serial_norm_ms) if a.no_overlap
+                                           else time_steps(grp, True))
+    if check_timeouts():
         return 1
 
     # ---- isolated kernels, HIP events on the launch stream -----------------------
     def time_kernel(fn, iters):
         """Average launch duration: `iters` back-to-back launches between one HIP event pair on
         the launch stream (what a kernel trace reports as the kernel's average), and the
-        shortest single launch out of 10 individually bracketed ones."""
-        e0, e1 = C.c_void_p(), C.c_void_p()
-        capi.check(L.fo_event_create(C.byref(e0)))
-        capi.check(L.fo_event_create(C.byref(e1)))
-        v = C.c_float()
-        for _ in range(5):
-            fn()
+        shortest single launch out of 10 individually bracketed ones.  fn takes the launch index."""
+        e0, e1 = tm.event(), tm.event()
+        for i in range(5):
+            fn(i)
         torch.cuda.synchronize()
-        capi.check(L.fo_event_record(e0, main_stream))
-        for _ in range(iters):
-            fn()
-        capi.check(L.fo_event_record(e1, main_stream))
+        tm.record(e0)
+        for i in range(iters):
+            fn(i)
+        tm.record(e1)
         torch.cuda.synchronize()
-        capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(v)))
-        avg = v.value / iters
+        avg = tm.ms(e0, e1) / iters
         best = float("inf")
-        for _ in range(10):
-            capi.check(L.fo_event_record(e0, main_stream))
-            fn()
-            capi.check(L.fo_event_record(e1, main_stream))
+        for i in range(10):
+            tm.record(e0)
+            fn(i)
+            tm.record(e1)
             torch.cuda.synchronize()
-            capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(v)))
-            best = min(best, v.value)
-        capi.check(L.fo_event_destroy(e0))
-        capi.check(L.fo_event_destroy(e1))
+            best = min(best, tm.ms(e0, e1))
+        tm.free(e0, e1)
         return avg, best
 
     it = a.kernel_iters
     # no waiter runs here: the group counters simply accumulate and are cleared afterwards
-    sig_ms, sig_min = time_kernel(gemm_signal, it)
-    MM.zero_()
-    pl_ms, pl_min = time_kernel(gemm_plain, it)
-    rms_ms, rms_min = time_kernel(norm, it)
+    sig_ms, sig_min = time_kernel(lambda i: gemm_signal(grp), it)
+    grp.MM.zero_()
+    pl_ms, pl_min = time_kernel(lambda i: gemm_plain(), it)
+    rms_rot_ms, _ = time_kernel(lambda i: norm(i % npairs), it)      # rotation larger than the memory-side cache
+    rms_same_ms, rms_min = time_kernel(lambda i: norm(0), it)         # one pair over and over: served by that cache
     cons_ms, _ = time_kernel(
-        lambda: capi.check(L.fo_consume(Cp.data_ptr(), staging.data_ptr(), 2 * M * N, main_stream)), it)
+        lambda i: capi.check(L.fo_consume(Cp.data_ptr(), stagings[i % npairs].data_ptr(), 2 * M * N, main_stream)), it)
+    # The same instruction stream on all-zero operands: the MFMAs toggle nothing, the chip stays
+    # below its power limit and keeps its clock.  What separates this figure from gemm_plain is
+    # the power limit, not the kernel's schedule.
+    A0, B0 = torch.zeros_like(A), torch.zeros_like(B)
+    z_ms, _ = time_kernel(lambda i: gemm_plain(A0, B0), max(10, it // 4))
+    del A0, B0
+
+    other = None
+    if a.both_readings and a.workload in WAVE_READING and not a.group_tiles:
+        w2 = w_tiles if w == w_waves else w_waves
+        g2 = Grouping(w2)
+        s2_serial, _, _ = time_steps(g2, False)
+        s2_ms, s2_gemm, _ = (s2_serial, 0.0, 0.0) if a.no_overlap else time_steps(g2, True)
+        if check_timeouts():
+            return 1
+        sig2_ms, _ = time_kernel(lambda i: gemm_signal(g2), it)
+        g2.MM.zero_()
+        other = {"reading": "waves" if w2 == w_waves else "tiles", "tiles_per_group": w2, "groups": g2.G,
+                 "consumer": consumer_name(g2), "ms_per_step": round(s2_ms, 5), "serial_step_ms": round(s2_serial, 5),
+                 "gemm_signal_in_step_us": round(s2_gemm * 1e3, 2), "gemm_signal_isolated_us": round(sig2_ms * 1e3, 2),
+                 "signal_overhead_pct": round((sig2_ms / pl_ms - 1.0) * 100.0, 2)}
 
     flops = 2.0 * M * N * K
     rms_bytes = 2.0 * (M * N * 2) + N * 2
     cons_bytes = 2.0 * (M * N * 2)
     sig_tf = flops / sig_ms / 1e9
     pl_tf = flops / pl_ms / 1e9
-    rms_gbps = rms_bytes / rms_ms / 1e6
-    cu, khz, xcd = C.c_int(), C.c_int(), C.c_int()
-    capi.check(L.fo_device_info(C.byref(cu), C.byref(khz), C.byref(xcd)))
-
     # ---- CPU baseline: the oracle on a bounded sample of the same workload -------
     cpu = None
     if a.cpu_seconds > 0:
@@ -284,14 +360,20 @@ def main() -> int:
                          f"({best[0]:.2f} s, matmul {best[1]:.2f} s)",
                "host_cpus": os.cpu_count()}
 
+    def hbm(ms):
+        gbps = rms_bytes / ms / 1e6
+        return {"achieved": round(gbps, 1), "frac": round(gbps / PEAK_HBM_GBPS, 4), "avg_us": round(ms * 1e3, 2)}
+
+    reading = ("tiles" if w == w_tiles else "waves" if w == w_waves else "custom") if a.workload in WAVE_READING else "waves"
     line = {
         "metric": "signaling-GEMM TFLOP/s", "value": round(flops / step_ms / 1e9, 2), "unit": "TFLOP/s",
+        "value_is": "2*M*N*K / whole step time (signalling GEMM || consumer, then reorder+RMSNorm); "
+                    "the GEMM kernel's own rate is roofline.achieved",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(step_ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dts, "data": "synthetic",
         "config": {"workload": f"{a.workload}: {NAMES[a.workload]}", "M": M, "N": N, "K": K,
-                   "layout_tile": [BM, BN], "tiles": T, "tiles_per_wave": TILES_PER_WAVE, "tiles_per_group": w, "groups": G, "world_size": ws,
-                   "eps": eps, "consumer": ("one wait kernel + one copy launch per group" if per_group else
-                                f"persistent wait+consume, {a.consumer_blocks} workgroups"),
+                   "layout_tile": [BM, BN], "tiles": T, "tiles_per_wave": TILES_PER_WAVE, "group_size_reading": reading,
+                   "tiles_per_group": w, "groups": grp.G, "world_size": ws, "eps": eps, "consumer": consumer_name(grp),
                    "step": ("signal GEMM -> wait+consume -> reorder+RMSNorm (serial)" if a.no_overlap else
                             "signal GEMM || wait+consume -> join -> reorder+RMSNorm")},
         "serial_step_ms": round(serial_ms, 5),
@@ -304,20 +386,27 @@ def main() -> int:
                      "launches": a.steps},
         "gemm_signal_serial_step": {"achieved": round(flops / serial_gemm_ms / 1e9, 2), "unit": "TFLOP/s",
                                     "avg_us": round(serial_gemm_ms * 1e3, 2)},
-        # the same kernel launched back to back on its own (A and B stay in the 256 MB Infinity Cache)
+        # the same kernel launched back to back on its own (A and B stay in the 256 MB memory-side cache)
         "gemm_signal_isolated": {"achieved": round(sig_tf, 2), "unit": "TFLOP/s",
                                  "frac": round(sig_tf / PEAK_MFMA_TFLOPS, 4), "avg_us": round(sig_ms * 1e3, 2),
                                  "min_us": round(sig_min * 1e3, 2), "launches": it},
         "cpu_baseline": cpu,
         "gemm_plain": {"achieved": round(pl_tf, 2), "unit": "TFLOP/s", "frac": round(pl_tf / PEAK_MFMA_TFLOPS, 4),
                        "avg_us": round(pl_ms * 1e3, 2), "min_us": round(pl_min * 1e3, 2)},
+        "gemm_plain_zero_operands": {"achieved": round(flops / z_ms / 1e9, 2), "unit": "TFLOP/s",
+                                     "frac": round(flops / z_ms / 1e9 / PEAK_MFMA_TFLOPS, 4),
+                                     "avg_us": round(z_ms * 1e3, 2),
+                                     "note": "same kernel and shape, A = B = 0: not power-limited"},
         "signal_overhead_pct": round((sig_ms / pl_ms - 1.0) * 100.0, 2),
-        "reorder_rmsnorm": {"bound": "hbm", "achieved": round(rms_gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                            "frac": round(rms_gbps / PEAK_HBM_GBPS, 4), "avg_us": round(rms_ms * 1e3, 2),
-                            "min_us": round(rms_min * 1e3, 2), "bytes": rms_bytes},
+        # headline: back to back over a rotation of buffer pairs that exceeds the memory-side cache
+        "reorder_rmsnorm": {"bound": "hbm", "peak": PEAK_HBM_GBPS, "unit": "GB/s", "bytes": rms_bytes,
+                            **hbm(rms_rot_ms), "buffer_pairs": npairs,
+                            "in_step": hbm(step_norm_ms),
+                            "same_pair_back_to_back": {**hbm(rms_same_ms), "min_us": round(rms_min * 1e3, 2)}},
         "consume_copy": {"achieved": round(cons_bytes / cons_ms / 1e6, 1), "unit": "GB/s",
                          "avg_us": round(cons_ms * 1e3, 2)},
-        "device": {"cu": cu.value, "clock_khz": khz.value, "xcd": xcd.value},
+        "other_reading": other,
+        "device": {"cu": cu.value, "clock_khz": khz.value, "xcd_assumed": xcd.value},
     }
     print(json.dumps(line))
     return 0

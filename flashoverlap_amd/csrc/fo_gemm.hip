@@ -31,8 +31,14 @@
 // tile-permuted layout, optionally with the row index mapped through RE
 // (scatter).  Then the signal: after every wavefront's stores have been
 // acknowledged and the workgroup has met at a barrier, one lane per layout
-// tile bumps the tile's group counter with a release-ordered, agent-scope
-// atomic.  The plain GEMM is the same kernel with the signalling compiled out.
+// tile bumps the tile's group counter with an agent-scope atomic.  The tile
+// stores are agent-scope write-through stores (sc1), the instruction the
+// compiler emits for an agent-scope atomic store: once s_waitcnt vmcnt(0)
+// returns they have been performed at agent scope, so nothing dirty is left in
+// this XCD's L2 for a release to write back, and the counter atomic can be a
+// relaxed one.  (The release-ordered form, cached stores or not, is kept as a
+// tuning knob: its buffer_wbl2 costs 3-10 % of a short-K GEMM.)  The plain
+// GEMM is the same kernel with the signalling compiled out.
 //
 // Semantics follow the reference epilogues src/overlap/gemm_with_signal.h:145-201
 // and src/overlap/gemm_with_scatter.h:146-196; the kernel itself shares nothing
@@ -81,7 +87,7 @@ enum { kPlain = 0, kSignal = 1, kScatter = 2 };
 
 // Tuning knobs (fo_tune): how the epilogue stores C and how it signals.
 int g_store_mode = 1;    // 0 = cached stores, 1 = agent-scope write-through stores (sc1)
-int g_release_mode = 0;  // 0 = release-ordered atomic, 1 = write-through stores + relaxed atomic (needs store mode 1)
+int g_release_mode = 1;  // 1 = write-through tile stores, acknowledged, then a relaxed atomic; 0 = release-ordered atomic
 
 struct GemmParams {
     const void* A;
@@ -427,9 +433,10 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 
     // ---- signal ---------------------------------------------------------------------
     if constexpr (MODE != kPlain) {
-        // Every wave's tile stores are acknowledged before the barrier; the
-        // release on the atomic then makes them visible device-wide before
-        // the counter moves.
+        // Every wave's tile stores are acknowledged before the barrier: with
+        // write-through stores they are then visible device-wide (REL = 1);
+        // otherwise the release on the atomic writes this L2's dirty lines back
+        // before the counter moves.
         wait_vmcnt<0>();
         __syncthreads();
         const int ntile = (MT / p.BM) * (MT / p.BN);

@@ -15,6 +15,8 @@
 // hang the device.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "fo_internal.h"
 
 namespace fo {
@@ -48,31 +50,33 @@ __global__ void wait_kernel(int that, int* addr, long long ticks) {
         atomicAdd(&g_wait_timeouts, 1);
 }
 
-constexpr int kCopyThreads = 512;  // consumer workgroup size
+constexpr int kCopyThreads = 512;  // workgroup size of the per-group copy kernel
 constexpr int kCopyUnroll = 8;     // 16-byte units in flight per thread
-constexpr long long kUnitsPerTeamMember = 8192;  // 128 KiB: what one workgroup takes of a group before another joins
+constexpr int kWavesPerBlock = 4;  // persistent consumer: one wavefront per SIMD
+constexpr long long kUnitsPerMember = 2048;  // 32 KiB: what one wavefront takes of a group before another joins
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // Copies n 16-byte units (n * 16 < 4 GiB) as member `me` of a team of `team`
-// workgroups, which interleave in chunks of kCopyThreads * kCopyUnroll units,
-// every thread keeping kCopyUnroll loads in flight.  COHERENT: read with
-// agent-scope loads that do not hit in the non-coherent caches (for data
-// another XCD wrote while this kernel runs).  All accesses are non-temporal:
-// the copy streams through and must not push the GEMM's operands out of the
-// 256 MB memory-side cache, from which the next GEMM's L2 misses are served
-// (with ordinary accesses here the next GEMM ran 10-15 % slower).
-template <bool COHERENT>
+// members of WIDTH threads each (`t` is the thread's index inside its member),
+// which interleave in chunks of WIDTH * kCopyUnroll units, every thread keeping
+// kCopyUnroll loads in flight.  COHERENT: read with agent-scope loads that do
+// not hit in the non-coherent caches (for data another XCD wrote while this
+// kernel runs).  All accesses are non-temporal: the copy streams through and
+// must not push the GEMM's operands out of the 256 MB memory-side cache, from
+// which the next GEMM's L2 misses are served (with ordinary accesses here the
+// next GEMM ran 10-15 % slower).
+template <bool COHERENT, int WIDTH>
 __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __restrict__ d, long long n, int me,
-                                          int team) {
-    const long long chunk = (long long)kCopyThreads * kCopyUnroll;
+                                          int team, int t) {
+    const long long chunk = (long long)WIDTH * kCopyUnroll;
     [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc;
     if constexpr (COHERENT) rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, 0xffffffff, 0x00020000);
     for (long long base = (long long)me * chunk; base < n; base += (long long)team * chunk) {
         u32x4 v[kCopyUnroll];
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
-            const long long i = base + u * kCopyThreads + threadIdx.x;
+            const long long i = base + u * WIDTH + t;
             if (i < n) {
                 if constexpr (COHERENT) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(i * 16), 0, 16 | 2);  // sc1 nt
                 else v[u] = __builtin_nontemporal_load((const u32x4*)(s + i));
@@ -80,137 +84,108 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
         }
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
-            const long long i = base + u * kCopyThreads + threadIdx.x;
+            const long long i = base + u * WIDTH + t;
             if (i < n) __builtin_nontemporal_store(v[u], (u32x4*)(d + i));
         }
     }
 }
 
 // Persistent form of the host loop in src/overlap_impl.cu:257-265 (and
-// :312-323 for the ReduceScatter receive layout).  Every workgroup walks the
-// groups in index order.  A group is handled by a team of workgroups whose
-// size grows with the group (one member per 128 KiB, at most the whole grid);
-// the teams of consecutive groups are consecutive windows of the grid, so many
-// small groups are spread over the workgroups and one large group is copied by
-// all of them.  A member waits for the group's count, bumps MM[g] once more
-// (the member that brings it to cSeg[g] + team is the last to have seen the
-// count and stores the 0) and copies its stripe of the range.  With the whole
-// grid on every group the groups are released strictly in index order;
-// smaller teams release groups as they complete.  A group's range is cut into
-// nslices equal parts;
-// parts slice_first .. slice_first+slice_count-1 are copied, part k to
+// :312-323 for the ReduceScatter receive layout).  The members of the kernel
+// are its wavefronts; every member walks the groups in index order.  A group
+// is handled by a team of members whose size grows with the group (one member
+// per 32 KiB, at most all of them); the teams of consecutive groups are
+// consecutive windows of the member list, so many small groups are spread over
+// the members and one large group is copied by all of them.  A member waits
+// for the group's count, bumps MM[g] once more (the member that brings it to
+// cSeg[g] + team is the last to have seen the count and stores the 0) and
+// copies its stripe of the range.  With every member on every group the groups
+// are released strictly in index order; smaller teams release groups as they
+// complete.  A group's range is cut into nslices equal parts; parts
+// slice_first .. slice_first+slice_count-1 are copied, part k to
 // dst + (k - slice_first)*stride + offset/nslices (the receive layout of a
-// ReduceScatter; nslices = 1 is the plain copy).  The kernel needs few
-// registers and next to no LDS, so its waves fit beside a resident GEMM
-// workgroup on the same CU.
-__global__ void __launch_bounds__(kCopyThreads) wait_consume_kernel(const int* __restrict__ cseg, int G, int* MM,
-                                                                    const uint4* __restrict__ src,
-                                                                    uint4* __restrict__ dst, long long tile_units,
-                                                                    int nslices, int slice_first, int slice_count,
-                                                                    long long slice_stride_units, int* order_log,
-                                                                    long long ticks) {
-    // The groups are taken kCopyThreads at a time: one thread per group works out
-    // where the group starts and which window of the grid is its team (two block
-    // scans), the groups this workgroup belongs to are compacted into a list in
-    // index order, and the list is then worked off.
-    __shared__ int s_ok[2];
-    __shared__ long long s_units[kCopyThreads];
-    __shared__ int s_team[kCopyThreads];
-    __shared__ int s_pos[kCopyThreads];
-    __shared__ long long s_lo[kCopyThreads];
-    __shared__ int s_g[kCopyThreads], s_me[kCopyThreads], s_tm[kCopyThreads];
-    const int tid = threadIdx.x;
-    const int nb = gridDim.x;
+// ReduceScatter; nslices = 1 is the plain copy).
+//
+// The kernel uses no LDS and no workgroup barrier, and few registers: the GEMM
+// workgroup that runs on the same CU owns all of its LDS and most of its
+// registers, and these wavefronts have to fit beside it.  Each wavefront finds
+// its groups on its own: 64 groups at a time, one per lane, with wavefront
+// scans for the group offsets and the team windows.
+__global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
+    const int* __restrict__ cseg, int G, int* MM, const uint4* __restrict__ src, uint4* __restrict__ dst,
+    long long tile_units, int nslices, int slice_first, int slice_count, long long slice_stride_units,
+    int* order_log, long long ticks) {
+    const int lane = threadIdx.x & 63;
+    const int self = __builtin_amdgcn_readfirstlane((int)blockIdx.x * kWavesPerBlock + (int)(threadIdx.x >> 6));
+    const int members = (int)gridDim.x * kWavesPerBlock;
     long long lo_base = 0;  // first 16-byte unit of the chunk's first group
-    int start_base = 0;     // first workgroup of that group's team
-    int mine = 0;           // groups this workgroup has taken part in
-    for (int g0 = 0; g0 < G; g0 += kCopyThreads) {
-        const int g = g0 + tid;
-        long long units = 0;
+    int start_base = 0;     // first member of that group's team
+    for (int g0 = 0; g0 < G; g0 += 64) {
+        const int g = g0 + lane;
+        const int count = g < G ? cseg[g] : 0;
+        const long long units = tile_units * count;
         int team = 0;
         if (g < G) {
-            units = tile_units * cseg[g];
-            const long long want = (units + kUnitsPerTeamMember - 1) / kUnitsPerTeamMember;
-            team = (int)(want < 1 ? 1 : (want > nb ? nb : want));
+            const long long want = (units + kUnitsPerMember - 1) / kUnitsPerMember;
+            team = (int)(want < 1 ? 1 : (want > members ? members : want));
         }
-        // inclusive scans of units and team sizes over the chunk
-        s_units[tid] = units;
-        s_team[tid] = team;
-        __syncthreads();
-        for (int off = 1; off < kCopyThreads; off <<= 1) {
-            const long long u = tid >= off ? s_units[tid - off] : 0;
-            const int t = tid >= off ? s_team[tid - off] : 0;
-            __syncthreads();
-            s_units[tid] += u;
-            s_team[tid] += t;
-            __syncthreads();
-        }
-        const long long lo = lo_base + s_units[tid] - units;
-        const int start = (int)(((long long)start_base + s_team[tid] - team) % nb);
-        int me = (int)blockIdx.x - start;   // the team is a window of the grid
-        if (me < 0) me += nb;
-        const int own = (g < G && me < team) ? 1 : 0;
-        // compaction: position of every owned group in the list
-        s_pos[tid] = own;
-        __syncthreads();
-        for (int off = 1; off < kCopyThreads; off <<= 1) {
-            const int c = tid >= off ? s_pos[tid - off] : 0;
-            __syncthreads();
-            s_pos[tid] += c;
-            __syncthreads();
-        }
-        const int count = s_pos[kCopyThreads - 1];
-        const long long chunk_units = s_units[kCopyThreads - 1];
-        const int chunk_team = s_team[kCopyThreads - 1];
-        if (own) {
-            const int at = s_pos[tid] - 1;
-            s_g[at] = g;
-            s_me[at] = me;
-            s_tm[at] = team;
-            s_lo[at] = lo;
-        }
-        __syncthreads();
-        for (int i = 0; i < count; ++i) {
-            const int gg = s_g[i], tm = s_tm[i], mem = s_me[i];
-            const long long glo = s_lo[i];
-            const int need = cseg[gg];
-            int* ok_flag = s_ok + (mine++ & 1);   // two flags in turn: lane 0 may already be polling the next group
-            if (tid == 0) {
-                const bool ok = bounded_poll(MM + gg, ticks, [need](int v) { return v >= need; });
-                if (!ok) atomicAdd(&g_wait_timeouts, 1);
-                *ok_flag = ok;
+        // inclusive scans of units and team sizes over the 64 groups of the chunk
+        long long su = units;
+        int st = team;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const long long u = __shfl_up(su, off, 64);
+            const int t = __shfl_up(st, off, 64);
+            if (lane >= off) {
+                su += u;
+                st += t;
             }
-            __syncthreads();
-            if (!*ok_flag) return;  // uniform: the whole workgroup leaves
-            if (tid == 0) {
-                // Every member has seen the full count once it has bumped it; the last one
-                // to do so puts the counter back.  The copies need not be finished for that:
-                // the next writer of the counter is ordered behind this kernel.
-                bool last = tm == 1;
-                if (!last)
-                    last = __hip_atomic_fetch_add(MM + gg, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                           need + tm - 1;
-                if (last) {
-                    __hip_atomic_store(MM + gg, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (order_log) order_log[gg] = gg;
+        }
+        const long long lo = lo_base + su - units;
+        const int start = (int)(((long long)start_base + st - team) % members);
+        int me = self - start;   // the team is a window of the member list
+        if (me < 0) me += members;
+        unsigned long long mine = __ballot(g < G && me < team);
+        while (mine) {   // wave-uniform: the groups this wavefront belongs to, in index order
+            const int b = __builtin_ctzll(mine);
+            mine &= mine - 1;
+            const int gg = g0 + b;
+            const int tm = __shfl(team, b, 64), mem = __shfl(me, b, 64), need = __shfl(count, b, 64);
+            const long long glo = __shfl(lo, b, 64);
+            int ok = 0;
+            if (lane == 0) {
+                ok = bounded_poll(MM + gg, ticks, [need](int v) { return v >= need; }) ? 1 : 0;
+                if (!ok) {
+                    atomicAdd(&g_wait_timeouts, 1);
+                } else {
+                    // Every member has seen the full count once it has bumped it; the last one
+                    // to do so puts the counter back.  The copies need not be finished for that:
+                    // the next writer of the counter is ordered behind this kernel.
+                    bool last = tm == 1;
+                    if (!last)
+                        last = __hip_atomic_fetch_add(MM + gg, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                               need + tm - 1;
+                    if (last) {
+                        __hip_atomic_store(MM + gg, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (order_log) order_log[gg] = gg;
+                    }
                 }
             }
-            const long long gunits = tile_units * need;
-            const long long part = gunits / nslices;
+            if (!__shfl(ok, 0, 64)) return;  // the wait expired: this wavefront gives up on the rest
+            const long long part = tile_units * need / nslices;
             for (int k = 0; k < slice_count; ++k)
-                team_copy<true>(src + glo + (slice_first + k) * part, dst + k * slice_stride_units + glo / nslices,
-                                part, mem, tm);
+                team_copy<true, 64>(src + glo + (slice_first + k) * part, dst + k * slice_stride_units + glo / nslices,
+                                    part, mem, tm, lane);
         }
-        __syncthreads();   // the list is rewritten for the next chunk
-        lo_base += chunk_units;
-        start_base = (int)(((long long)start_base + chunk_team) % nb);
+        lo_base += __shfl(su, 63, 64);
+        start_base = (int)(((long long)start_base + __shfl(st, 63, 64)) % members);
     }
 }
 
 __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                                long long units, const unsigned short* src_tail,
                                                                unsigned short* dst_tail, int tail) {
-    team_copy<false>(src, dst, units, blockIdx.x, gridDim.x);
+    team_copy<false, kCopyThreads>(src, dst, units, blockIdx.x, gridDim.x, threadIdx.x);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
@@ -245,12 +220,34 @@ __global__ void __launch_bounds__(1024) group_table_kernel(const int* __restrict
     for (int s = total + tid; s < T; s += 1024) table[s] = G - 1;
 }
 
-static int ticks_for_timeout(long long* ticks) {
-    int dev = 0, khz = 0;
+// Per-device facts the launchers need on every call, looked up once per device.
+struct DeviceFacts {
+    int wall_khz = 0;   // rate of wall_clock64()
+    int cus = 0;
+};
+static int device_facts(const DeviceFacts** out) {
+    static DeviceFacts facts[64];
+    static std::atomic<unsigned long long> known{0};
+    int dev = 0;
     FO_HIP(hipGetDevice(&dev));
-    FO_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
-    if (khz <= 0) khz = 100000;  // the constant 100 MHz counter of gfx9
-    *ticks = (long long)g_timeout_ms * khz;
+    if (dev < 0 || dev >= 64) return fail(FO_ERR_LIMIT, "device %d beyond 64", dev);
+    const unsigned long long bit = 1ull << dev;
+    if (!(known.load(std::memory_order_acquire) & bit)) {
+        DeviceFacts f;
+        FO_HIP(hipDeviceGetAttribute(&f.wall_khz, hipDeviceAttributeWallClockRate, dev));
+        if (f.wall_khz <= 0) f.wall_khz = 100000;  // the constant 100 MHz counter of gfx9
+        FO_HIP(hipDeviceGetAttribute(&f.cus, hipDeviceAttributeMultiprocessorCount, dev));
+        facts[dev] = f;   // racing threads write the same values
+        known.fetch_or(bit, std::memory_order_release);
+    }
+    *out = &facts[dev];
+    return FO_OK;
+}
+
+static int ticks_for_timeout(long long* ticks) {
+    const DeviceFacts* f;
+    if (int e = device_facts(&f)) return e;
+    *ticks = (long long)g_timeout_ms * f->wall_khz;
     return FO_OK;
 }
 
@@ -285,15 +282,21 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
                         int nblocks, hipStream_t stream) {
     if (!cseg || !MM || !src || !dst) return fail(FO_ERR_ARG, "fo_wait_consume: null argument");
     if (G <= 0 || nslices <= 0 || tile_elems <= 0) return fail(FO_ERR_ARG, "fo_wait_consume: G=%d nslices=%d tile_elems=%lld", G, nslices, tile_elems);
-    if (nblocks <= 0 || nblocks > 1024) return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d outside 1..1024", nblocks);
+    if (nblocks <= 0) return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d", nblocks);
     if (tile_elems % (8LL * nslices)) return fail(FO_ERR_SHAPE, "fo_wait_consume: a tile (%lld elements) must split into %d slices of whole 16-byte units", tile_elems, nslices);
     if (slice_first < 0 || slice_count <= 0 || slice_first + slice_count > nslices)
         return fail(FO_ERR_ARG, "fo_wait_consume: slices [%d, %d) outside 0..%d", slice_first, slice_first + slice_count, nslices);
     if (slice_count > 1 && slice_stride % 8) return fail(FO_ERR_SHAPE, "fo_wait_consume: slice_stride=%lld not a multiple of 8 elements", slice_stride);
     if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_wait_consume: buffers must be 16-byte aligned");
+    // The workgroups wait while GEMM workgroups still have to be placed: at most one per CU, so that
+    // a consumer that is dispatched first can never keep a GEMM workgroup from fitting.
+    const DeviceFacts* facts;
+    if (int e = device_facts(&facts)) return e;
+    if (nblocks > facts->cus)
+        return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d outside 1..%d (one workgroup per CU)", nblocks, facts->cus);
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
-    hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(kCopyThreads), 0, stream, cseg, G, MM, (const uint4*)src,
+    hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(64 * kWavesPerBlock), 0, stream, cseg, G, MM, (const uint4*)src,
                        (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks);
     FO_HIP(hipGetLastError());
     return FO_OK;

@@ -43,8 +43,48 @@ void OverlapImpl::SetConsumerMode(int64_t mode) {
 }
 
 void OverlapImpl::SetConsumerBlocks(int64_t blocks) {
-    TORCH_CHECK(blocks >= 1 && blocks <= 1024, "set_consumer_blocks: 1..1024, got ", blocks);
+    int cus = 0;
+    FO_CALL(fo_device_info(&cus, nullptr, nullptr));
+    // The persistent consumer's workgroups wait beside the GEMM's: at most one per CU.
+    TORCH_CHECK(blocks >= 1 && blocks <= cus, "set_consumer_blocks: 1..", cus, " (one workgroup per CU), got ", blocks);
     consumer_blocks_ = blocks;
+}
+
+int OverlapImpl::consumer_blocks() {
+    if (consumer_blocks_ == 0) {   // default: one workgroup per CU
+        int cus = 0;
+        FO_CALL(fo_device_info(&cus, nullptr, nullptr));
+        consumer_blocks_ = cus;
+    }
+    return (int)consumer_blocks_;
+}
+
+void OverlapImpl::SetWaitTimeoutMs(int64_t ms) {
+    TORCH_CHECK(ms >= 1 && ms <= 3600 * 1000, "set_wait_timeout_ms: 1..3600000, got ", ms);
+    FO_CALL(fo_set_wait_timeout_ms((int)ms));
+}
+
+int64_t OverlapImpl::WaitTimeouts(bool reset) {
+    int n = 0;
+    FO_CALL(fo_wait_timeouts(&n, reset ? 1 : 0));
+    return n;
+}
+
+void OverlapImpl::SetCheckTimeouts(bool on) { check_timeouts_ = on; }
+
+// Checked mode: wait for the call to finish and turn an expired wait into an
+// error.  The counters then hold partial counts, which would make every later
+// wait on them expire too (or pass at once), so they are cleared here.
+void OverlapImpl::raise_on_timeout(at::Tensor& MM, const char* who) {
+    if (!check_timeouts_) return;
+    FO_CALL(fo_stream_sync(gemm_stream_));
+    int n = 0;
+    FO_CALL(fo_wait_timeouts(&n, 1));
+    if (n == 0) return;
+    MM.zero_();
+    TORCH_CHECK(false, who, ": ", n, " bounded wait(s) expired before their group completed; the consumer's output "
+                "is incomplete and MM has been zeroed (a cSeg that does not match the tiles, or a GEMM slower than the "
+                "wait timeout)");
 }
 
 at::Tensor OverlapImpl::Staging() const {
@@ -105,7 +145,7 @@ void OverlapImpl::consume_groups(const at::Tensor& C, void* dst, int64_t tile_el
     const bool persistent = consumer_mode_ == 2 || (consumer_mode_ == 0 && G > 32);
     if (persistent) {
         FO_CALL(fo_wait_consume(cseg_gpu.data_ptr<int>(), G, MM.data_ptr<int>(), C.data_ptr(), dst, tile_elems,
-                                nslices, slice_first, slice_count, slice_stride, nullptr, (int)consumer_blocks_,
+                                nslices, slice_first, slice_count, slice_stride, nullptr, consumer_blocks(),
                                 comm_stream_));
         return;
     }
@@ -141,6 +181,7 @@ void OverlapImpl::GemmAllReduceOverlap(at::Tensor A, at::Tensor B, at::Tensor C,
     // The caller's stream continues only after the last group is consumed
     // (src/overlap_impl.cu:267-270).
     FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
+    raise_on_timeout(MM, "gemm_allreduce_overlap");
 }
 
 void OverlapImpl::GemmReduceScatterOverlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor D, at::Tensor MM,
@@ -166,6 +207,7 @@ void OverlapImpl::GemmReduceScatterOverlap(at::Tensor A, at::Tensor B, at::Tenso
     const int64_t stride = (D.numel() == total && my_size_ > 1) ? total / my_size_ : 0;
     consume_groups(C, D.data_ptr(), (int64_t)g.BM * g.BN, cSEG_CPU, cSEG_GPU, MM, (int)my_size_, stride);
     FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
+    raise_on_timeout(MM, "gemm_reducescatter_overlap");
 }
 
 void OverlapImpl::GemmAllReduce(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo) {

@@ -53,8 +53,17 @@ class OverlapImpl : public torch::CustomClassHolder {
     // beyond), 1 = one (wait, consume) launch pair per group like the
     // reference's host loop, 2 = one persistent wait+consume kernel.
     void SetConsumerMode(int64_t mode);
-    // Workgroups of the persistent consumer (default 64).
+    // Workgroups of the persistent consumer (default and maximum: one per CU).
     void SetConsumerBlocks(int64_t blocks);
+    // The waits on the group counters are bounded (the reference's spin forever,
+    // src/wait.cuh:6-8).  set_wait_timeout_ms sets the bound (process-wide, default
+    // 10 s); wait_timeouts(reset) synchronises the device and returns how many
+    // waits have expired on it; set_check_timeouts(true) makes every overlapped call
+    // wait for its own completion and raise if one of its waits expired (debugging:
+    // it serialises the caller).  After an expiry MM must be zeroed before reuse.
+    void SetWaitTimeoutMs(int64_t ms);
+    int64_t WaitTimeouts(bool reset);
+    void SetCheckTimeouts(bool on);
 
   private:
     void* gemm_stream_ = nullptr;
@@ -63,7 +72,8 @@ class OverlapImpl : public torch::CustomClassHolder {
     int64_t my_rank_ = 0;
     int64_t my_size_ = 1;
     int64_t consumer_mode_ = 0;
-    int64_t consumer_blocks_ = 64;
+    int64_t consumer_blocks_ = 0;   // 0: not chosen yet (one per CU at first use)
+    bool check_timeouts_ = false;
 
     at::Tensor staging_;
     at::Tensor group_table_;
@@ -76,4 +86,6 @@ class OverlapImpl : public torch::CustomClassHolder {
     void consume_groups(const at::Tensor& C, void* dst, int64_t tile_elems, const at::Tensor& cseg_cpu,
                         const at::Tensor& cseg_gpu, at::Tensor& MM, int nslices, int64_t slice_stride);
     void bulk_consume(const void* src, void* dst, size_t bytes);
+    void raise_on_timeout(at::Tensor& MM, const char* who);
+    int consumer_blocks();
 };

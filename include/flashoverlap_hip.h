@@ -53,7 +53,10 @@ const char* fo_last_error(void);
 int fo_algo_count(void);
 int fo_algo_tile(int algo, int* BM, int* BN, int* BK);
 
-/* Device facts used for roofline reports: CU count, clock (kHz), XCD count. */
+/* Device facts used for roofline reports: CU count and clock (kHz) as HIP
+ * reports them.  xcd_count is not read from the device (HIP has no attribute
+ * for it): it is the constant 8 that the workgroup rasterisation of the GEMM
+ * is built for (MI355X: 8 accelerator dies of 32 CUs). */
 int fo_device_info(int* cu_count, int* clock_khz, int* xcd_count);
 
 /* ---- GEMM ------------------------------------------------------------- */
@@ -124,11 +127,14 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host);
 
 /* Process-wide tuning knobs of the GEMM epilogue, for measurement; no
  * counterpart in the reference.  Results are identical for every setting.
- *   "store_mode"   0: cached tile stores; 1: agent-scope write-through tile
- *                  stores (default: the release then finds no dirty lines to
- *                  write back).
- *   "release_mode" 0: release-ordered signal atomic (default); 1: write-through
- *                  tile stores, wait for their acknowledgement, relaxed atomic. */
+ *   "release_mode" 1 (default): the tile stores are agent-scope write-through
+ *                  stores; every wave waits for their acknowledgement, the
+ *                  workgroup meets at a barrier, then a relaxed agent-scope
+ *                  atomic bumps the counter.  0: a release-ordered atomic
+ *                  instead (L2 write-back first), with the tile stores as
+ *                  "store_mode" says.
+ *   "store_mode"   with release_mode 0 only.  1 (default): write-through tile
+ *                  stores; 0: cached tile stores. */
 int fo_tune(const char* key, int value);
 
 /* ---- counting / wait -------------------------------------------------- */
@@ -137,7 +143,10 @@ int fo_tune(const char* key, int value);
  * to *addr.  Replaces launch_kernel_wait_flag (src/wait_launch.h:5,
  * src/wait_launch.cu:5-7, kernel src/wait.cuh:5-9).  Unlike the reference the
  * wait is bounded (fo_set_wait_timeout_ms, default 10000 ms): on expiry the
- * kernel leaves *addr untouched, bumps the timeout count and returns. */
+ * kernel leaves *addr untouched, bumps the timeout count and returns; what
+ * follows on the stream then works on an incomplete group, so a caller checks
+ * fo_wait_timeouts at its next synchronisation point and zeroes MM after an
+ * expiry. */
 int fo_wait(int that, int* addr, void* stream);
 
 /* One persistent kernel in place of G (wait, collective) launch pairs: for
@@ -151,11 +160,16 @@ int fo_wait(int that, int* addr, void* stream);
  * src/overlap_impl.cu:257-265); nslices == world size with one slice is what a
  * rank receives from the per-group ReduceScatter (src/overlap_impl.cu:312-323),
  * with all slices it is every rank's receive buffer side by side.
- * Of the nblocks workgroups a team of one per 128 KiB of the group (at most
- * all) handles a group; consecutive groups go to consecutive teams.  Groups of
- * nblocks x 128 KiB and more are therefore released strictly in index order by
- * the whole grid, smaller ones as they complete.  order_log (optional, G ints)
- * gets order_log[g] = g when group g has been released and its counter reset. */
+ * The kernel runs nblocks workgroups of four wavefronts (1 <= nblocks <= CU
+ * count; it uses no LDS and few registers, so a workgroup fits beside a GEMM
+ * workgroup on a CU).  Of the 4 * nblocks wavefronts a team of one per 32 KiB
+ * of the group (at most all) handles a group; consecutive groups go to
+ * consecutive teams.  Groups of nblocks x 128 KiB and more are therefore
+ * released strictly in index order by the whole grid, smaller ones as they
+ * complete.  order_log (optional, G ints) gets order_log[g] = g when group g
+ * has been released and its counter reset.  If a wait expires the wavefront
+ * counts it (fo_wait_timeouts) and stops; MM then holds partial counts and
+ * must be zeroed by the caller before it is used again. */
 int fo_wait_consume(const int* cseg_dev, int G, int* MM,
                     const void* src, void* dst, long long tile_elems,
                     int nslices, int slice_first, int slice_count, long long slice_stride,

@@ -1,5 +1,5 @@
 """The persistent consumer on its own: ragged group sizes (zeros included) over
-several 512-group passes, every counter preset to its group's size, for
+several 64-group passes, every counter preset to its group's size, for
 different grid sizes and with the ReduceScatter slicing; checked against the
 oracle's consume_allreduce / consume_reducescatter."""
 import ctypes as C
@@ -14,7 +14,7 @@ from oracle import fo_oracle as O
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("nblocks", [1, 7, 64, 300])
+@pytest.mark.parametrize("nblocks", [1, 7, 64, 256])
 @pytest.mark.parametrize("ws", [1, 4])
 def test_ragged_groups(fo_lib, dev, nblocks, ws):
     L = fo_lib
@@ -43,3 +43,16 @@ def test_ragged_groups(fo_lib, dev, nblocks, ws):
     else:
         want = O.consume_reducescatter(src, sizes, BM, BN, ws).reshape(-1)
     assert torch.equal(d_dst.cpu(), want)
+
+
+def test_more_workgroups_than_cus_is_refused(fo_lib, dev):
+    """The consumer's workgroups wait while GEMM workgroups still have to be placed, so there may be
+    at most one per CU; a larger grid is an error, not a silent clamp."""
+    L = fo_lib
+    cu = C.c_int()
+    capi.check(L.fo_device_info(C.byref(cu), None, None))
+    buf = torch.zeros(4096, dtype=torch.int32, device=dev)
+    rc = L.fo_wait_consume(buf.data_ptr(), 1, buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), 128, 1, 0, 1, 0, None,
+                           cu.value + 1, None)
+    assert rc == capi.FO_ERR_LIMIT
+    assert b"one workgroup per CU" in L.fo_last_error()

@@ -74,15 +74,15 @@ class Path:
                                   self.dB.data_ptr(), out.data_ptr(), stream))
         return out
 
-    def gemm_signal(self, use_table=True, stream=None):
+    def gemm_signal(self, use_table=True, stream=None, rldn=1):
         table = self.dtable.data_ptr() if use_table else None
-        if self.ws > 1:
-            capi.check(self.L.fo_gemm_scatter(self.code, self.algo, self.M, self.N, self.K, 1, self.dcseg.data_ptr(),
+        if self.dRE is not None:
+            capi.check(self.L.fo_gemm_scatter(self.code, self.algo, self.M, self.N, self.K, rldn, self.dcseg.data_ptr(),
                                               self.G, table, self.dA.data_ptr(), self.dB.data_ptr(),
                                               self.dC.data_ptr(), self.dMM.data_ptr(), self.dRA.data_ptr(),
                                               self.dRE.data_ptr(), int(self.monitor), stream))
         else:
-            capi.check(self.L.fo_gemm_signal(self.code, self.algo, self.M, self.N, self.K, 1, self.dcseg.data_ptr(),
+            capi.check(self.L.fo_gemm_signal(self.code, self.algo, self.M, self.N, self.K, rldn, self.dcseg.data_ptr(),
                                              self.G, table, self.dA.data_ptr(), self.dB.data_ptr(),
                                              self.dC.data_ptr(), self.dMM.data_ptr(), self.dRA.data_ptr(),
                                              int(self.monitor), stream))
@@ -189,6 +189,64 @@ def test_signal_placement_counters_and_table(L, dev, dt, M, N, K, algo, w):
     torch.cuda.synchronize()
     assert p.dMM.cpu()[:p.G].tolist() == p.cseg
     assert torch.equal(p.dC.cpu(), O.place_tiles(natural.cpu(), p.ra_host.numpy(), BM, BN, 1))
+
+
+@pytest.mark.parametrize("dt,M,N,K,algo", [(torch.float16, 512, 1024, 128, 1), (torch.bfloat16, 1024, 512, 64, 1),
+                                           (torch.bfloat16, 512, 1024, 64, 3), (torch.float16, 2048, 4096, 64, 1)])
+def test_signal_rldn_tn_identity_equals_plain_gemm(L, dev, dt, M, N, K, algo):
+    """rLDN = TN with the identity RA makes the permuted view the natural row-major [M, N]
+    (src/overlap/gemm_with_signal.h:149-165): the signalling kernel, and the scatter kernel with an
+    identity RE, must then write exactly what the plain GEMM writes."""
+    _say("signal rLDN=TN identity", dt, M, N, K, algo)
+    BM, BN, _ = capi.algo_tile(algo)
+    TN = N // BN
+    T = (M // BM) * TN
+    p = Path(L, dev, dt, M, N, K, algo, cseg=O.uniform_cseg(T, 3), hint=list(range(T)), seed=11)
+    assert p.ra_host.tolist() == list(range(T))
+    p.build_table()
+    natural = p.gemm_plain()
+    p.gemm_signal(rldn=TN)
+    torch.cuda.synchronize()
+    assert torch.equal(p.dC.view(M, N), natural)
+    assert p.dMM.cpu()[:p.G].tolist() == p.cseg
+    # scatter kernel, identity row map
+    p.dRE = torch.arange(M * N // BN, dtype=torch.int32, device=dev)
+    p.dC.zero_()
+    p.dMM.zero_()
+    p.gemm_signal(rldn=TN)
+    torch.cuda.synchronize()
+    assert torch.equal(p.dC.view(M, N), natural)
+    assert p.dMM.cpu()[:p.G].tolist() == p.cseg
+
+
+@pytest.mark.parametrize("dt,M,N,K,algo,rldn", [(torch.float16, 512, 1024, 128, 1, 2), (torch.bfloat16, 1024, 1024, 64, 1, 4),
+                                                (torch.bfloat16, 1024, 2048, 64, 3, 2), (torch.float16, 2048, 2048, 64, 5, 8),
+                                                (torch.bfloat16, 2048, 4096, 64, 1, 16)])
+def test_signal_and_scatter_general_rldn(L, dev, dt, M, N, K, algo, rldn):
+    """rLDN > 1 with a random RA (and, for the scatter kernel, a random row permutation RE of the
+    [M*N/(rLDN*BN), rLDN*BN] view) against the oracle's epilogues, bit-exact."""
+    _say("signal rLDN", dt, M, N, K, algo, rldn)
+    BM, BN, _ = capi.algo_tile(algo)
+    T = (M // BM) * (N // BN)
+    rng = np.random.default_rng(rldn * 31 + algo)
+    p = Path(L, dev, dt, M, N, K, algo, cseg=O.uniform_cseg(T, 5), hint=rng.permutation(T).tolist(),
+             integer_inputs=True, seed=rldn)
+    p.build_table()
+    p.gemm_signal(rldn=rldn)
+    torch.cuda.synchronize()
+    natural = O.gemm(p.A, p.B)
+    assert torch.equal(p.dC.cpu(), O.place_tiles(natural, p.ra_host.numpy(), BM, BN, rldn))
+    assert p.dMM.cpu()[:p.G].tolist() == p.cseg
+    rows = M * N // (rldn * BN)                      # rows of the permuted view
+    re = np.arange(M * N // BN, dtype=np.int32)
+    re[:rows] = rng.permutation(rows).astype(np.int32)
+    p.dRE = torch.from_numpy(re).to(dev)
+    p.dC.zero_()
+    p.dMM.zero_()
+    p.gemm_signal(rldn=rldn)
+    torch.cuda.synchronize()
+    assert torch.equal(p.dC.cpu(), O.scatter_place(natural, p.ra_host.numpy(), re, BM, BN, rldn))
+    assert p.dMM.cpu()[:p.G].tolist() == p.cseg
 
 
 def test_group_table_edge_cases(L, dev):
