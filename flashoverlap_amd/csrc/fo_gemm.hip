@@ -3,7 +3,15 @@
 //
 // One workgroup of 4 wavefronts computes one MT x MT macro tile (MT = 256, or
 // 128 for small problems); each wavefront owns an (MT/2) x (MT/2) quadrant as
-// (MT/64)^2 blocks of v_mfma_f32_32x32x16, accumulators in AGPRs.
+// (MT/32)^2 blocks of v_mfma_f32_16x16x32, accumulators in AGPRs.  The 16x16x32
+// form reads and writes a quarter of the accumulator registers per flop of the
+// 32x32x16 form (the k-reduction of 32 happens inside the instruction); the
+// chip runs this kernel at its power limit, and the kernel measured 3-4 %
+// faster with it.  The MFMAs are issued through inline assembly with the
+// accumulators pinned to AGPRs: with the compiler builtin the register
+// allocator moved 16x16 accumulators between the two register files inside
+// the main loop.  The order of the main loop's instructions is therefore
+// written out slot by slot in the source and fenced, not left to the scheduler.
 //
 // Main loop: A and B panels of 64 k-elements stream HBM -> LDS with
 // buffer_load_dwordx4 ... lds (no register staging) into a ring of five panel
@@ -14,9 +22,10 @@
 // this tile size the kernel sits at the edge of that request rate, so half-line
 // requests cost a quarter of the throughput.  The 16-byte chunks of a row are
 // XOR-swizzled by row so the ds_read_b128 fragment reads are bank-conflict
-// free.  A k-step of 64 is four quarter steps of 16 MFMAs each; the fragments
-// of all four are read during the first two, so while one quarter's MFMAs run
-// the fragments of the next are already in registers, and the workgroup
+// free.  A k-step of 64 is four quarter steps of 32 MFMAs each (two per k half
+// of 32); the fragments of all four are read during the first two, so while
+// one quarter's MFMAs run the fragments of the next are already in registers,
+// and the workgroup
 // barrier that releases the panel's two slots sits in the middle of the
 // k-step.  The free slot lets the copies of A(p+2) go out in the first half of
 // k-step p and those of B(p+2) in the second half: the same number of copies
@@ -59,6 +68,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T>
@@ -67,16 +77,16 @@ template <>
 struct Mma<_Float16> {
     using frag = f16x8;
     using out4 = f16x4;
-    static __device__ __forceinline__ f32x16 run(frag a, frag b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    static __device__ __forceinline__ void run(frag a, frag b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 template <>
 struct Mma<__bf16> {
     using frag = bf16x8;
     using out4 = bf16x4;
-    static __device__ __forceinline__ f32x16 run(frag a, frag b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    static __device__ __forceinline__ void run(frag a, frag b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 
@@ -139,16 +149,26 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 template <int N>
 using template_int = std::integral_constant<int, N>;
 
+// f(integral_constant<0>) ... f(integral_constant<N-1>)
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(template_int<N - 1>{});
+    }
+}
+
 // STORE: 0 cached, 1 write-through tile stores; REL: 0 release atomic, 1 relaxed atomic.
 template <typename T, int MT, int MODE, int STORE, int REL>
 __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     constexpr int WT = MT / 2;               // wave quadrant edge
-    constexpr int NB = WT / 32;              // 32x32 MFMA blocks per quadrant edge
+    constexpr int NB = WT / 16;              // 16x16 MFMA blocks per quadrant edge
+    constexpr int NH = NB / 2;               // A blocks per quarter step
     constexpr int PANEL = MT * kRowBytes;    // bytes of one A (or B) panel = one LDS slot
     constexpr int LOADS = MT / 32;           // wave-wide 1 KiB copies per wave per panel
     constexpr int LPT = 2 * LOADS;           // copies per wave per k-step
     constexpr int HALF = LPT / 2;
-    constexpr int BLK = 32 * kRowBytes;      // LDS bytes between 32-row blocks
+    constexpr int BLK = 16 * kRowBytes;      // LDS bytes between 16-row blocks
     using frag = typename Mma<T>::frag;
     using out4 = typename Mma<T>::out4;
 
@@ -238,67 +258,40 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     std::true_type unit_b;
 
     // ---- LDS -> register fragment addressing ----------------------------------
-    // MFMA 32x32x16 operand: lane l supplies row l%32, k = 8*(l/32) .. +7.
-    const int fr_row = lane & 31, fr_h = lane >> 5;
+    // MFMA 16x16x32 operand: lane l supplies row l%16, k = 8*(l/16) .. +7 of a k half.
+    const int fr_row = lane & 15, fr_h = lane >> 4;
     const int a_lane = (wm * WT + fr_row) * kRowBytes;
     const int b_lane = (wn * WT + fr_row) * kRowBytes;
-    int ko[4];   // chunk offset of each quarter step (k 0..15, 16..31, 32..47, 48..63)
+    int ko[2];   // chunk offset of each k half (k 0..31, 32..63)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) ko[q] = ((2 * q + fr_h) ^ swz(fr_row)) * 16;
+    for (int h = 0; h < 2; ++h) ko[h] = ((4 * h + fr_h) ^ swz(fr_row)) * 16;
 
-    f32x16 acc[NB][NB];
+    f32x4 acc[NB][NB];
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+            for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
 
-    // Fragments of the four quarter steps of a panel (k 0..15, 16..31, 32..47, 48..63).
-    frag fa[4][NB], fb[4][NB];
+    // Fragments of the two k halves of a panel.  Quarter step q works on k half
+    // q/2 and on the A blocks (q%2)*NH .. +NH: its own A fragments and, in the
+    // first quarter of a half, all B fragments of the half.
+    frag fa[2][NB], fb[2][NB];
 
     auto load_frags = [&](int slot_a, int slot_b, int q) {
-        const unsigned char* pa = smem + slot_a + ko[q] + a_lane;
-        const unsigned char* pb = smem + slot_b + ko[q] + b_lane;
+        const int h = q >> 1, i0 = (q & 1) * NH;
+        const unsigned char* pa = smem + slot_a + ko[h] + a_lane;
+        const unsigned char* pb = smem + slot_b + ko[h] + b_lane;
 #pragma unroll
-        for (int i = 0; i < NB; ++i) fa[q][i] = *(const frag*)(pa + i * BLK);
+        for (int i = i0; i < i0 + NH; ++i) fa[h][i] = *(const frag*)(pa + i * BLK);
+        if ((q & 1) == 0) {
 #pragma unroll
-        for (int j = 0; j < NB; ++j) fb[q][j] = *(const frag*)(pb + j * BLK);
-    };
-    // Operands swapped (B rows as the MFMA "A" matrix) so that a lane ends up
-    // with 4 consecutive n for one m.
-    auto mma = [&](int q) {
-#pragma unroll
-        for (int i = 0; i < NB; ++i)
-#pragma unroll
-            for (int j = 0; j < NB; ++j) acc[i][j] = Mma<T>::run(fb[q][j], fa[q][i], acc[i][j]);
-    };
-    // Scheduling hint for one quarter step of NB*NB MFMAs: LDS reads go out one
-    // per MFMA at the front, so that the MFMAs behind them cover their latency
-    // and the wait at the end of the quarter does not stall; the HBM->LDS copies
-    // follow, one per MFMA.
-    auto interleave = [&](auto reads_c, auto copies_c) {
-        constexpr int reads = decltype(reads_c)::value;
-        constexpr int copies = decltype(copies_c)::value;
-        constexpr int NM = NB * NB;
-#pragma unroll
-        for (int slot = 0; slot < reads && slot < NM; ++slot) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one DS read
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+            for (int j = 0; j < NB; ++j) fb[h][j] = *(const frag*)(pb + j * BLK);
         }
-        if constexpr (copies > 0 && reads < NM) {
-            constexpr int per_slot = (copies + (NM - reads) - 1) / (NM - reads);
-#pragma unroll
-            for (int i = 0; i < copies; i += per_slot) {
-                __builtin_amdgcn_sched_group_barrier(0x020, per_slot, 0);  // VMEM reads
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            }
-        } else if constexpr (copies > 0) {
-            __builtin_amdgcn_sched_group_barrier(0x020, copies, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, NM, 0);  // whatever MFMAs are left
     };
-    constexpr int FR = 2 * NB;   // LDS reads per quarter's fragments
+    constexpr int FR0 = NH + NB;  // LDS reads for the first quarter of a k half (A blocks + all B blocks)
+    constexpr int FR1 = NH;       // for the second quarter
     template_int<0> first_half;
     template_int<1> second_half;
     auto end_quarter = [&](auto pending_reads_c) {
@@ -317,21 +310,62 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     // during the second half.
     // NEXT: panel kt+1 exists.  C2: panel kt+2 exists.
     constexpr int QC = LOADS / 2;   // copies per quarter per wave
+    // One copy instruction (slab j of the A or B unit of panel kt) into slot `slot`.
+    auto issue_one = [&](int kt, int slot, auto isb_c, auto j_c) {
+        constexpr bool ISB = decltype(isb_c)::value;
+        constexpr int j = decltype(j_c)::value;
+        unsigned char* dst = smem + slot + lds_cp;
+        const unsigned koff = (unsigned)kt * (kBK * 2);
+        const int voff = (j & 1) ? cp_off1 : cp_off0;
+        if constexpr (ISB)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, voff,
+                                                     (int)(baseB + j * slab_bytes + koff), 0, 0);
+        else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(dst + j * 1024), 16, voff,
+                                                     (int)(baseA + j * slab_bytes + koff), 0, 0);
+    };
+    // One fragment read.
+    auto read_a = [&](int slot_a, int h, int i) { fa[h][i] = *(const frag*)(smem + slot_a + ko[h] + a_lane + i * BLK); };
+    auto read_b = [&](int slot_b, int h, int j) { fb[h][j] = *(const frag*)(smem + slot_b + ko[h] + b_lane + j * BLK); };
+    constexpr int NM = NH * NB;   // MFMAs per quarter step
+    // A quarter step, written out slot by slot: before MFMA s go read `s` of the
+    // quarter's read list (reader(s)) and, if a copy is due, one copy; nothing is
+    // allowed to move across a slot boundary.
+    auto quarter = [&](auto q_c, auto nreads_c, auto reader, auto ncopies_c, auto copier) {
+        constexpr int q = decltype(q_c)::value;
+        constexpr int nreads = decltype(nreads_c)::value;
+        constexpr int ncopies = decltype(ncopies_c)::value;
+        constexpr int h = q >> 1, i0 = (q & 1) * NH;
+        constexpr int cstart = nreads < NM - 2 * ncopies ? nreads : NM - 2 * ncopies;   // copies every other slot
+        static_for<NM>([&](auto s_c) {
+            constexpr int sl = decltype(s_c)::value;
+            if constexpr (sl < nreads) reader(s_c);
+            if constexpr (ncopies > 0 && sl >= cstart && ((sl - cstart) & 1) == 0 && (sl - cstart) / 2 < ncopies)
+                copier(template_int<(sl - cstart) / 2>{});
+            __builtin_amdgcn_sched_barrier(0);
+            // operands swapped (B rows as the MFMA "A" matrix): a lane ends up with 4 consecutive n for one m
+            Mma<T>::run(fb[h][sl % NB], fa[h][i0 + sl / NB], acc[i0 + sl / NB][sl % NB]);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
     auto kstep = [&](int kt, int sa, int sb, int na, int nb, int sp, auto next_c, auto c2_c) {
         constexpr bool NEXT = decltype(next_c)::value;
         constexpr bool C2 = decltype(c2_c)::value;
-        // quarter 0: fragments of quarters 1 and 2 go out, only quarter 1's are awaited
-        load_frags(sa, sb, 1);
-        load_frags(sa, sb, 2);
-        if constexpr (C2) issue_unit(kt + 2, sp, unit_a, first_half);
-        mma(0);
-        interleave(template_int<2 * FR>{}, template_int<(C2 ? QC : 0)>{});
-        end_quarter(template_int<FR>{});
-        // quarter 1: fragments of quarter 3
-        load_frags(sa, sb, 3);
-        if constexpr (C2) issue_unit(kt + 2, sp, unit_a, second_half);
-        mma(1);
-        interleave(template_int<FR>{}, template_int<(C2 ? QC : 0)>{});
+        // quarter 0 (k half 0, A blocks 0..NH-1): reads for quarter 1 (A blocks NH.. of half 0), then
+        // for quarter 2 (A blocks 0..NH-1 and all B blocks of half 1); first half of A(kt+2)
+        quarter(template_int<0>{}, template_int<FR1 + FR0>{},
+                [&](auto r_c) {
+                    constexpr int r = decltype(r_c)::value;
+                    if constexpr (r < NH) read_a(sa, 0, NH + r);
+                    else if constexpr (r < 2 * NH) read_a(sa, 1, r - NH);
+                    else read_b(sb, 1, r - 2 * NH);
+                },
+                template_int<(C2 ? QC : 0)>{}, [&](auto c_c) { issue_one(kt + 2, sp, unit_a, c_c); });
+        end_quarter(template_int<FR0>{});
+        // quarter 1: reads for quarter 3 (A blocks NH.. of half 1); second half of A(kt+2)
+        quarter(template_int<1>{}, template_int<FR1>{}, [&](auto r_c) { read_a(sa, 1, NH + decltype(r_c)::value); },
+                template_int<(C2 ? QC : 0)>{},
+                [&](auto c_c) { issue_one(kt + 2, sp, unit_a, template_int<QC + decltype(c_c)::value>{}); });
         end_quarter(template_int<0>{});
         if constexpr (NEXT) {
             // Panel kt+1 has landed for every wave (the copies of A(kt+2), the newest
@@ -342,15 +376,18 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
             __builtin_amdgcn_sched_barrier(0);
         }
         // quarter 2: first half of B(kt+2) into the slot A(kt) just left
-        if constexpr (C2) issue_unit(kt + 2, sa, unit_b, first_half);
-        mma(2);
-        interleave(template_int<0>{}, template_int<(C2 ? QC : 0)>{});
+        quarter(template_int<2>{}, template_int<0>{}, [&](auto) {}, template_int<(C2 ? QC : 0)>{},
+                [&](auto c_c) { issue_one(kt + 2, sa, unit_b, c_c); });
         end_quarter(template_int<0>{});
-        // quarter 3: first fragments of panel kt+1, second half of B(kt+2)
-        if constexpr (NEXT) load_frags(na, nb, 0);
-        if constexpr (C2) issue_unit(kt + 2, sa, unit_b, second_half);
-        mma(3);
-        interleave(template_int<(NEXT ? FR : 0)>{}, template_int<(C2 ? QC : 0)>{});
+        // quarter 3: fragments of the first quarter of panel kt+1, second half of B(kt+2)
+        quarter(template_int<3>{}, template_int<(NEXT ? FR0 : 0)>{},
+                [&](auto r_c) {
+                    constexpr int r = decltype(r_c)::value;
+                    if constexpr (r < NH) read_a(na, 0, r);
+                    else read_b(nb, 0, r - NH);
+                },
+                template_int<(C2 ? QC : 0)>{},
+                [&](auto c_c) { issue_one(kt + 2, sa, unit_b, template_int<QC + decltype(c_c)::value>{}); });
         end_quarter(template_int<0>{});
     };
 
@@ -393,7 +430,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     kstep(kt, sa, sb, na, nb, sp, std::false_type{}, std::false_type{});
 
     // ---- epilogue: registers -> LDS strip -> global -------------------------------
-    // acc[i][j][4q+r] is element m = 32i + l%32, n = 32j + 8q + 4(l/32) + r.
+    // acc[i][j][r] is element m = 16i + l%16, n = 16j + 4(l/16) + r.
     __builtin_amdgcn_s_setprio(0);
     __syncthreads();  // every wave is done with the panel buffers
     constexpr int PITCH = WT * 2 + 16;                  // strip row pitch in bytes
@@ -403,15 +440,15 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     [[maybe_unused]] __amdgpu_buffer_rsrc_t drsrc;
     if constexpr (STORE == 1) drsrc = __builtin_amdgcn_make_buffer_rsrc(p.D, 0, 0xffffffff, 0x00020000);
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
+    for (int i = 0; i < NB / 2; ++i) {   // strip i: rows 32i .. 32i+31 of the quadrant
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
+        for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+            for (int j = 0; j < NB; ++j) {
                 out4 o;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = (T)acc[i][j][4 * q + r];
-                *(out4*)(ep + fr_row * PITCH + (32 * j + 8 * q + 4 * fr_h) * 2) = o;
+                for (int r = 0; r < 4; ++r) o[r] = (T)acc[2 * i + ii][j][r];
+                *(out4*)(ep + (16 * ii + fr_row) * PITCH + (16 * j + 4 * fr_h) * 2) = o;
             }
 #pragma unroll
         for (int it = 0; it < WT / 16; ++it) {

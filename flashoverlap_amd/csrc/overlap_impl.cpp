@@ -92,6 +92,14 @@ at::Tensor OverlapImpl::Staging() const {
     return staging_;
 }
 
+void OverlapImpl::SetStaging(at::Tensor buffer) {
+    TORCH_CHECK(buffer.defined() && buffer.is_cuda() && buffer.is_contiguous(),
+                "set_staging: the buffer must be a contiguous GPU tensor");
+    TORCH_CHECK(buffer.scalar_type() == at::kHalf || buffer.scalar_type() == at::kBFloat16,
+                "set_staging: the buffer must be float16 or bfloat16, got ", buffer.scalar_type());
+    staging_ = buffer.view({buffer.numel()});
+}
+
 void OverlapImpl::require_gemm() const {
     TORCH_CHECK(gemm_ready_, "OverlapImpl: call mutlass_init() first");
 }

@@ -49,6 +49,11 @@ class OverlapImpl : public torch::CustomClassHolder {
     // Destination of the AllReduce stand-in: a flat buffer of the size of the
     // last C passed to an all-reduce style call.
     at::Tensor Staging() const;
+    // Makes `buffer` (M*N elements of C's dtype) the destination of the next
+    // all-reduce style calls instead of the internally allocated one, so that a
+    // caller can own its result like it owns C in the reference.  A call whose C
+    // does not match the buffer in size, dtype or device goes back to an internal one.
+    void SetStaging(at::Tensor buffer);
     // 0 = automatic (per-group launches up to 32 groups, one persistent kernel
     // beyond), 1 = one (wait, consume) launch pair per group like the
     // reference's host loop, 2 = one persistent wait+consume kernel.

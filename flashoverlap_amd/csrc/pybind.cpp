@@ -55,6 +55,7 @@ TORCH_LIBRARY(flashoverlap_class, m) {
         // additions
         .def("staging", &OverlapImpl::Staging)
         .def("set_consumer_mode", &OverlapImpl::SetConsumerMode)
+        .def("set_staging", &OverlapImpl::SetStaging)
         .def("set_consumer_blocks", &OverlapImpl::SetConsumerBlocks)
         .def("set_wait_timeout_ms", &OverlapImpl::SetWaitTimeoutMs)
         .def("wait_timeouts", &OverlapImpl::WaitTimeouts)

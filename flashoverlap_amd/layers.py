@@ -63,9 +63,10 @@ class OverlapRowParallelLayer(nn.Module):
     """The overlapped linear of example/RowParallelLinear.py:35-85 on one GPU.
 
     config: dict with BM, BN, Algo, hint, cSeg (flashoverlap_amd.config).
-    all_reduce returns the staging buffer (tile-permuted, feed it to
-    ReorderRMSNorm); reduce_scatter returns this rank's receive buffer
-    [M/world_size, N] (normalise it with BM // world_size).
+    all_reduce returns a fresh tile-permuted tensor (feed it to
+    ReorderRMSNorm) that the caller owns, like `out` in the reference;
+    reduce_scatter returns this rank's receive buffer [M/world_size, N]
+    (normalise it with BM // world_size).
     """
 
     def __init__(self, rank: int, world_size: int, in_features: int, out_features: int, M: int, config: dict,
@@ -93,10 +94,13 @@ class OverlapRowParallelLayer(nn.Module):
     def forward(self, x):
         n = self.weight.size(0)
         if self.comm_op == "all_reduce":
+            # tmp receives the GEMM's tiles; the per-group copies (the collective's stand-in) land in out
+            tmp = torch.empty((x.size(0), n), dtype=x.dtype, device=x.device)
             out = torch.empty((x.size(0), n), dtype=x.dtype, device=x.device)
-            self.overlap_class.gemm_allreduce_overlap(x, self.weight, out, self.counter, self.reorder_array, 1,
+            self.overlap_class.set_staging(out)
+            self.overlap_class.gemm_allreduce_overlap(x, self.weight, tmp, self.counter, self.reorder_array, 1,
                                                       self.cseg_cpu, self.cseg_gpu, self.algo, False)
-            return self.overlap_class.staging().view(x.size(0), n)
+            return out
         tmp = torch.empty((x.size(0), n), dtype=x.dtype, device=x.device)
         out = torch.empty((x.size(0) // self.world_size, n), dtype=x.dtype, device=x.device)
         self.overlap_class.gemm_reducescatter_overlap(x, self.weight, tmp, out, self.counter, self.reorder_array,

@@ -53,8 +53,13 @@ def test_allreduce_layers_like_correctness_ar(ready, tmp_path):
     olin.weight = torch.nn.Parameter(B)
     with torch.no_grad():
         y1 = norm(lin(A))
-        y2 = rnorm(olin(A))
+        x2 = olin(A)
+        y2 = rnorm(x2)
+        # the layer's result belongs to the caller: a second forward must not overwrite it
+        kept = x2.clone()
+        x3 = olin(torch.zeros_like(A))
     torch.cuda.synchronize()
+    assert x3.data_ptr() != x2.data_ptr() and torch.equal(x2, kept) and not x3.any()
     assert _no_timeouts()
     assert torch.allclose(y1, y2, atol=1e-2, rtol=1e-2)                       # the reference's bar
     ref = O.rmsnorm(O.gemm(A.cpu(), B.cpu()), W.cpu(), 1e-5)
