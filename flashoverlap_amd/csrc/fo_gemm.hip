@@ -258,13 +258,19 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     std::true_type unit_b;
 
     // ---- LDS -> register fragment addressing ----------------------------------
-    // MFMA 16x16x32 operand: lane l supplies row l%16, k = 8*(l/16) .. +7 of a k half.
-    const int fr_row = lane & 15, fr_h = lane >> 4;
+    // MFMA 16x16x32 operand: lane l supplies row l%16 and the 8 k-values of lane
+    // group l/16.  Which 8 of the k half's 32 a group takes is free as long as A
+    // and B agree; groups 0..3 take the 16-byte chunks 0, 2, 1, 3.  The LDS
+    // serves lanes l and l+32 in the same pass: this way the two read
+    // neighbouring chunks of one row, which the row swizzle keeps on different
+    // banks (chunks 0 and 2 of the same rows would collide two ways).
+    const int fr_row = lane & 15, fr_g = lane >> 4;
+    const int fr_kc = (fr_g & 1) * 2 + (fr_g >> 1);
     const int a_lane = (wm * WT + fr_row) * kRowBytes;
     const int b_lane = (wn * WT + fr_row) * kRowBytes;
     int ko[2];   // chunk offset of each k half (k 0..31, 32..63)
 #pragma unroll
-    for (int h = 0; h < 2; ++h) ko[h] = ((4 * h + fr_h) ^ swz(fr_row)) * 16;
+    for (int h = 0; h < 2; ++h) ko[h] = ((4 * h + fr_kc) ^ swz(fr_row)) * 16;
 
     f32x4 acc[NB][NB];
 #pragma unroll
@@ -430,7 +436,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     kstep(kt, sa, sb, na, nb, sp, std::false_type{}, std::false_type{});
 
     // ---- epilogue: registers -> LDS strip -> global -------------------------------
-    // acc[i][j][r] is element m = 16i + l%16, n = 16j + 4(l/16) + r.
+    // acc[i][j][r] is element m = 16i + l%16, n = 16j + 4(l/16) + r (fr_g = l/16).
     __builtin_amdgcn_s_setprio(0);
     __syncthreads();  // every wave is done with the panel buffers
     constexpr int PITCH = WT * 2 + 16;                  // strip row pitch in bytes
@@ -448,7 +454,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
                 out4 o;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) o[r] = (T)acc[2 * i + ii][j][r];
-                *(out4*)(ep + (16 * ii + fr_row) * PITCH + (16 * j + 4 * fr_h) * 2) = o;
+                *(out4*)(ep + (16 * ii + fr_row) * PITCH + (16 * j + 4 * fr_g) * 2) = o;
             }
 #pragma unroll
         for (int it = 0; it < WT / 16; ++it) {
@@ -477,11 +483,27 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         wait_vmcnt<0>();
         __syncthreads();
         const int ntile = (MT / p.BM) * (MT / p.BN);
-        if (tid < ntile) {
+        // The tiles of a macro tile mostly fall into one group: the first lane of
+        // every distinct group adds that group's tile count in one atomic (at most
+        // four lanes take part, all in the first wavefront).  Monitor mode keeps
+        // one atomic per tile, like the reference: the tickets are per tile.
+        int same = 0, earlier = 0;
+        if (wave == 0) {
+#pragma unroll
+            for (int o = 0; o < 4; ++o) {
+                const int g = __shfl(sig_group, o, 64);
+                if (o < ntile && g == sig_group) {
+                    ++same;
+                    if (o < tid) ++earlier;
+                }
+            }
+        }
+        if (tid < ntile && (p.monitor || earlier == 0)) {
+            const int add = p.monitor ? 1 : same;
             if constexpr (REL == 1)  // the stores already went through to memory
-                __hip_atomic_fetch_add(p.MM + sig_group, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(p.MM + sig_group, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             else
-                __hip_atomic_fetch_add(p.MM + sig_group, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(p.MM + sig_group, add, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
             if (p.monitor) {
                 const int order =
                     __hip_atomic_fetch_add(p.MM + p.TN - 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -27,6 +27,20 @@ def _say(*a):
     print(*a, flush=True)
 
 
+def _max_abs_ok(got, ref):
+    """max-abs 2e-2, except where that is less than two units in the last place of the storage
+    type.  The kernel's only freedom is the order of the fp32 accumulation, which can move an
+    element of C by one storage ulp; downstream that element is rounded twice more (scaled value,
+    then times gamma), so the final value can land two ulps from the oracle's.  A bf16 value of
+    magnitude 2..4 has ulp 2^-6: two of them are 0.031 > 2e-2, so from that magnitude on the bound
+    is two ulps."""
+    mant = 7 if ref.dtype == torch.bfloat16 else 10
+    r = ref.float().abs().clamp_min(2.0 ** -20)
+    ulp = torch.exp2(torch.floor(torch.log2(r)) - mant)
+    tol = torch.maximum(torch.full_like(ulp, MAX_ABS_TOL), 2 * ulp)
+    return bool(((got.float() - ref.float()).abs() <= tol).all())
+
+
 class Path:
     """One problem instance with its device buffers, driven through the C ABI."""
 
@@ -309,7 +323,7 @@ def test_scatter_epilogue_and_reducescatter_slices(L, dev, comm_stream, ws, cseg
         out = p.reorder_rmsnorm(D[k], 1e-5, bs=M // ws, BM=BM // ws)
         torch.cuda.synchronize()
         ref = O.rmsnorm(natural[k::ws], p.gamma, 1e-5)
-        assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and O.max_abs(out.cpu(), ref) < MAX_ABS_TOL
+        assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and _max_abs_ok(out.cpu(), ref)
     # one rank's view: only slice 1
     p.gemm_signal()
     one = torch.zeros(M * N // ws, dtype=p.dt, device=dev)
@@ -483,7 +497,7 @@ def _full_path(L, dev, comm_stream, dt, M, N, K, w, eps, ws=1, a_std=None, b_std
     unq = O.rmsnorm_fp32(c32, p.gamma, eps)
     _say("  vs unquantised fp32: rel-L2 %.2e max-abs %.2e" % (O.rel_l2(got, unq), O.max_abs(got, unq)))
     _say("  vs storage-matched : rel-L2 %.2e max-abs %.2e" % (O.rel_l2(got, gated), O.max_abs(got, gated)))
-    assert O.rel_l2(got, gated) < REL_L2_TOL and O.max_abs(got, gated) < MAX_ABS_TOL
+    assert O.rel_l2(got, gated) < REL_L2_TOL and _max_abs_ok(got, gated)
     # permutation invariants at full size: un-permuting the signalled output gives the plain kernel's output
     natural = p.gemm_plain()
     torch.cuda.synchronize()
