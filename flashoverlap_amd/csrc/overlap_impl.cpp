@@ -143,7 +143,8 @@ void OverlapImpl::Gemm(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo) {
 
 // Per-group release: either the reference's host loop (one wait kernel and one
 // consumer launch per group, src/overlap_impl.cu:257-265 / 312-323) or one
-// persistent kernel that does the same walk on the device.
+// persistent kernel that does the same walk on the device.  On return the GEMM
+// stream is ordered behind every group's copy.
 void OverlapImpl::consume_groups(const at::Tensor& C, void* dst, int64_t tile_elems, const at::Tensor& cseg_cpu,
                                  const at::Tensor& cseg_gpu, at::Tensor& MM, int nslices, int64_t slice_stride) {
     const int G = (int)cseg_cpu.numel();
@@ -155,18 +156,31 @@ void OverlapImpl::consume_groups(const at::Tensor& C, void* dst, int64_t tile_el
         FO_CALL(fo_wait_consume(cseg_gpu.data_ptr<int>(), G, MM.data_ptr<int>(), C.data_ptr(), dst, tile_elems,
                                 nslices, slice_first, slice_count, slice_stride, nullptr, consumer_blocks(),
                                 comm_stream_));
+        // The caller's stream continues only after the last group is consumed
+        // (src/overlap_impl.cu:267-270).
+        FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
         return;
     }
     const size_t esz = C.element_size();
     const char* src = (const char*)C.data_ptr();
     int64_t acc = 0;
     for (int g = 0; g < G; ++g) {
+        // The last group completes with the GEMM, so nothing is left for it to overlap with:
+        // it is released on the GEMM's own stream, behind the join of the groups before it.
+        // That join has been satisfied long before the stream reaches it, whereas a join
+        // behind the last group would put a fresh cross-stream dependency (10-20 us on this
+        // platform) between the last copy and the caller's next kernel.
+        void* stream = comm_stream_;
+        if (g == G - 1) {
+            if (G > 1) FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
+            stream = gemm_stream_;
+        }
         const int64_t comm = tile_elems * cseg[g];
-        FO_CALL(fo_wait(cseg[g], MM.data_ptr<int>() + g, comm_stream_));
+        FO_CALL(fo_wait(cseg[g], MM.data_ptr<int>() + g, stream));
         const int64_t part = comm / nslices;
         for (int k = 0; k < slice_count; ++k)
             FO_CALL(fo_consume(src + (acc + (slice_first + k) * part) * esz,
-                               (char*)dst + (k * slice_stride + acc / nslices) * esz, part * esz, comm_stream_));
+                               (char*)dst + (k * slice_stride + acc / nslices) * esz, part * esz, stream));
         acc += comm;
     }
 }
@@ -186,9 +200,6 @@ void OverlapImpl::GemmAllReduceOverlap(at::Tensor A, at::Tensor B, at::Tensor C,
                            A.data_ptr(), B.data_ptr(), C.data_ptr(), MM.data_ptr<int>(), RA.data_ptr<int>(),
                            if_monitor ? 1 : 0, gemm_stream_));
     consume_groups(C, staging.data_ptr(), (int64_t)g.BM * g.BN, cSEG_CPU, cSEG_GPU, MM, 1, 0);
-    // The caller's stream continues only after the last group is consumed
-    // (src/overlap_impl.cu:267-270).
-    FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
     raise_on_timeout(MM, "gemm_allreduce_overlap");
 }
 
@@ -214,7 +225,6 @@ void OverlapImpl::GemmReduceScatterOverlap(at::Tensor A, at::Tensor B, at::Tenso
                             RE.data_ptr<int>(), if_monitor ? 1 : 0, gemm_stream_));
     const int64_t stride = (D.numel() == total && my_size_ > 1) ? total / my_size_ : 0;
     consume_groups(C, D.data_ptr(), (int64_t)g.BM * g.BN, cSEG_CPU, cSEG_GPU, MM, (int)my_size_, stride);
-    FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
     raise_on_timeout(MM, "gemm_reducescatter_overlap");
 }
 

@@ -132,7 +132,15 @@ def perf_running(M, N, K, BM, BN, Algo, cSeg, hint, comm_op, world_size=1, dtype
         fn = lambda: o.gemm_reducescatter_overlap(A, B, C, D, counters, RA, RE, 1, cSeg_CPU, cSeg_GPU, Algo, False)
     dur = _timed(fn, **kw)
     if keep is not None:
-        keep.update(A=A, B=B, C=C, D=D, RA=RA, RE=RE, counters=counters, overlap=o)
+        # host time to enqueue one call (nothing is waited for): what the torch-API path costs the CPU
+        import time
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            fn()
+        host_us = (time.perf_counter() - t0) / 20 * 1e6
+        torch.cuda.synchronize()
+        keep.update(A=A, B=B, C=C, D=D, RA=RA, RE=RE, counters=counters, overlap=o, host_us_per_call=host_us)
     return dur
 
 
@@ -160,12 +168,13 @@ def speed_table(M, N, K, comm_op="all_reduce", cfg=None, world_size=1, dtype=tor
         data["hint"] = list(range(tile_num))
     mublas = perf_mublas_gemm(M, N, K, dtype, device, **kw)
     comm = perf_comm(M, N, comm_op, world_size, dtype, device, **kw)
+    keep = {} if keep is None else keep
     overlap = perf_running(M, N, K, data["BM"], data["BN"], data["Algo"], data["cSeg"], data["hint"], comm_op,
                            world_size, dtype, device, keep=keep, **kw)
     baseline = perf_baseline(M, N, K, comm_op, world_size, dtype, device, **kw)
     return {"m": M, "n": N, "k": K, "tile_num": tile_num, "cSeg": list(data["cSeg"]), "num_segs": len(data["cSeg"]),
             "mutlass_gemm": float(data["dur"]), "mublas_gemm": mublas, "mccl_comm": comm, "baseline": baseline,
-            "overlap": overlap, "speedup": baseline / overlap}
+            "overlap": overlap, "speedup": baseline / overlap, "overlap_host_us": keep["host_us_per_call"]}
 
 
 def format_table(t) -> str:
@@ -178,6 +187,7 @@ def format_table(t) -> str:
                        ("mccl_comm", "mccl_comm (ms)"), ("baseline", "baseline (mublas+mccl)"),
                        ("overlap", "overlap (mutlass+mccl)"), ("speedup", "speedup")):
         out.append(f"{label:<25} {t[key]:>15.4f}")
+    out.append(f"{'overlap host enqueue (us)':<25} {t['overlap_host_us']:>15.1f}")
     return "\n".join(out)
 
 

@@ -201,7 +201,9 @@ def test_expired_wait_is_reported_through_the_torch_api(api, dev):
     BM, BN, _ = capi.algo_tile(algo)
     TM, TN = M // BM, N // BN
     T = TM * TN
-    cSeg_CPU = torch.tensor([T], dtype=torch.int32)
+    # two groups: the first one (released on the second stream, where the wait starts with the GEMM)
+    # holds tiles of the GEMM's last round, so it completes only when the GEMM ends, after ~1.5 ms
+    cSeg_CPU = torch.tensor([T - 256, 256], dtype=torch.int32)
     cSeg_GPU = cSeg_CPU.to(dev)
     counter = torch.zeros(TN, dtype=torch.int32, device=dev)
     RA = tiling.reorder_indices(T, tiling.raster_hint(M, N, algo), dev).reshape(TM, TN)
