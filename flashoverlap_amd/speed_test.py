@@ -144,6 +144,54 @@ def perf_running(M, N, K, BM, BN, Algo, cSeg, hint, comm_op, world_size=1, dtype
     return dur
 
 
+def sustained_gemm(M, N, K, Algo=1, dtype=torch.float16, device="cuda", seconds=3.0, zeros=False):
+    """Both GEMMs in a loop of `seconds` each (launches are queued 200 at a time), with the core clock
+    sampled from rocm-smi while they run: what the chip sustains once its power management has
+    settled, as opposed to the bursts of a few milliseconds that the table times.  zeros=True runs
+    the same kernels on all-zero operands, which toggle nothing in the MFMA datapath.
+    Returns {name: (us_per_launch, [sclk MHz samples])}."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    import time
+    A, B, C = _operands(M, N, K, dtype, device)
+    if zeros:
+        A.zero_()
+        B.zero_()
+    o = _overlap_object()
+    b = torch.classes.flashoverlap_class.BaselineImpl()
+    b.mublas_init()
+    smi = shutil.which("rocm-smi")
+    out = {}
+    for name, fn in (("mutlass_gemm", lambda: o.mutlass_gemm(A, B, C, Algo)), ("mublas_gemm", lambda: b.mublas_gemm(A, B, C))):
+        clocks, stop = [], threading.Event()
+
+        def sample():
+            while smi and not stop.is_set():
+                try:
+                    txt = subprocess.run([smi, "--showclocks"], capture_output=True, text=True, timeout=5).stdout
+                    m = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", txt)
+                    if m:
+                        clocks.append(int(m.group(1)))
+                except Exception:
+                    pass
+                stop.wait(0.25)
+        th = threading.Thread(target=sample)
+        th.start()
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(200):
+                fn()
+            torch.cuda.synchronize()
+            n += 200
+        dt = time.perf_counter() - t0
+        stop.set()
+        th.join()
+        out[name] = (dt / n * 1e6, clocks)
+    return out
+
+
 def default_config(M, N, K, Algo=1, dtype=torch.float16, device="cuda", **kw):
     """A tuning record for a shape that has no file: this library's issue order as the hint, one
     hardware wave (256 macro tiles) per group, the measured plain-GEMM time as `dur`."""
@@ -202,6 +250,9 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", default="float16", choices=["float16", "bfloat16"])
     ap.add_argument("--configs", default="configs", help="directory of the per-shape tuning files")
     ap.add_argument("--save", action="store_true", help="write the tuning file if the shape has none")
+    ap.add_argument("--sustained", type=float, default=0.0,
+                    help="also loop each GEMM for this many seconds (random, then all-zero operands) and report "
+                         "the sustained time per launch and the core clock")
     ap.add_argument("--rep", type=int, default=REP)
     ap.add_argument("--warm_up", type=int, default=WARM_UP)
     a = ap.parse_args(argv)
@@ -222,6 +273,13 @@ def main(argv=None) -> int:
             config.save_solution(path, cfg["BM"], cfg["BN"], cfg["dur"], cfg["Algo"], cfg["hint"], cfg["cSeg"], 1)
     t = speed_table(m, n, k, a.comm_op, cfg, a.world_size, dtype, "cuda", a.single_seg, **kw)
     print(format_table(t))
+    if a.sustained > 0:
+        flops = 2.0 * m * n * k
+        for zeros in (False, True):
+            r = sustained_gemm(m, n, k, cfg["Algo"], dtype, "cuda", a.sustained, zeros)
+            for name, (us, clocks) in r.items():
+                print(f"sustained {a.sustained:.0f} s, {'zero' if zeros else 'random'} operands: {name:<13} {us:8.1f} us "
+                      f"{flops / us / 1e6:7.1f} TFLOP/s  sclk MHz {clocks[2:] if len(clocks) > 4 else clocks}")
     return 0
 
 
