@@ -96,6 +96,7 @@ constexpr int kRowBytes = kBK * 2;  // one panel row in LDS: 128 bytes = 8 chunk
 enum { kPlain = 0, kSignal = 1, kScatter = 2 };
 
 // Tuning knobs (fo_tune): how the epilogue stores C and how it signals.
+extern int g_copy_streaming_stores;   // fo_sync.hip
 int g_store_mode = 1;    // 0 = cached stores, 1 = agent-scope write-through stores (sc1)
 int g_release_mode = 1;  // 1 = write-through tile stores, acknowledged, then a relaxed atomic; 0 = release-ordered atomic
 
@@ -620,6 +621,7 @@ int tune(const char* key, int value) {
     const std::string_view k(key);
     if (k == "store_mode") g_store_mode = value ? 1 : 0;
     else if (k == "release_mode") g_release_mode = value ? 1 : 0;
+    else if (k == "copy_streaming_stores") g_copy_streaming_stores = value ? 1 : 0;
     else return fail(FO_ERR_ARG, "fo_tune: unknown knob '%s'", key);
     return FO_OK;
 }

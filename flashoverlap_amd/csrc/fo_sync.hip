@@ -24,6 +24,7 @@ namespace fo {
 __device__ int g_wait_timeouts = 0;
 
 static int g_timeout_ms = 10000;
+int g_copy_streaming_stores = 0;   // fo_tune "copy_streaming_stores": non-temporal stores in the consumer copy
 
 // Bounded poll of *addr until pred(value); returns false on expiry.
 template <typename Pred>
@@ -62,13 +63,15 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // which interleave in chunks of WIDTH * kCopyUnroll units, every thread keeping
 // kCopyUnroll loads in flight.  COHERENT: read with agent-scope loads that do
 // not hit in the non-coherent caches (for data another XCD wrote while this
-// kernel runs).  All accesses are non-temporal: the copy streams through and
-// must not push the GEMM's operands out of the 256 MB memory-side cache, from
-// which the next GEMM's L2 misses are served (with ordinary accesses here the
-// next GEMM ran 10-15 % slower).
+// kernel runs).  The loads are non-temporal: the source streams through once.
+// The stores are ordinary ones by default, so that the destination can stay in
+// the 256 MB memory-side cache for the kernel that reads it next (on some
+// machines reorder+RMSNorm took 30 us instead of 24 right behind a copy with
+// non-temporal stores); streaming_stores != 0 makes them non-temporal, which
+// keeps the copy from displacing other data in that cache.
 template <bool COHERENT, int WIDTH>
 __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __restrict__ d, long long n, int me,
-                                          int team, int t) {
+                                          int team, int t, int streaming_stores) {
     const long long chunk = (long long)WIDTH * kCopyUnroll;
     [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc;
     if constexpr (COHERENT) rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, 0xffffffff, 0x00020000);
@@ -85,7 +88,10 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
             const long long i = base + u * WIDTH + t;
-            if (i < n) __builtin_nontemporal_store(v[u], (u32x4*)(d + i));
+            if (i < n) {
+                if (streaming_stores) __builtin_nontemporal_store(v[u], (u32x4*)(d + i));
+                else *(u32x4*)(d + i) = v[u];
+            }
         }
     }
 }
@@ -114,7 +120,7 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
 __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
     const int* __restrict__ cseg, int G, int* MM, const uint4* __restrict__ src, uint4* __restrict__ dst,
     long long tile_units, int nslices, int slice_first, int slice_count, long long slice_stride_units,
-    int* order_log, long long ticks) {
+    int* order_log, long long ticks, int streaming_stores) {
     const int lane = threadIdx.x & 63;
     const int self = __builtin_amdgcn_readfirstlane((int)blockIdx.x * kWavesPerBlock + (int)(threadIdx.x >> 6));
     const int members = (int)gridDim.x * kWavesPerBlock;
@@ -175,7 +181,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
             const long long part = tile_units * need / nslices;
             for (int k = 0; k < slice_count; ++k)
                 team_copy<true, 64>(src + glo + (slice_first + k) * part, dst + k * slice_stride_units + glo / nslices,
-                                    part, mem, tm, lane);
+                                    part, mem, tm, lane, streaming_stores);
         }
         lo_base += __shfl(su, 63, 64);
         start_base = (int)(((long long)start_base + __shfl(st, 63, 64)) % members);
@@ -184,8 +190,8 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
 
 __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                                long long units, const unsigned short* src_tail,
-                                                               unsigned short* dst_tail, int tail) {
-    team_copy<false, kCopyThreads>(src, dst, units, blockIdx.x, gridDim.x, threadIdx.x);
+                                                               unsigned short* dst_tail, int tail, int streaming_stores) {
+    team_copy<false, kCopyThreads>(src, dst, units, blockIdx.x, gridDim.x, threadIdx.x, streaming_stores);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
@@ -297,7 +303,8 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
     hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(64 * kWavesPerBlock), 0, stream, cseg, G, MM, (const uint4*)src,
-                       (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks);
+                       (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks,
+                       g_copy_streaming_stores);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }
@@ -315,7 +322,7 @@ int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream)
     if (blocks == 0) blocks = 1;
     hipLaunchKernelGGL(consume_kernel, dim3((unsigned)blocks), dim3(kCopyThreads), 0, stream, (const uint4*)src,
                        (uint4*)dst, (long long)units, (const unsigned short*)((const char*)src + units * 16),
-                       (unsigned short*)((char*)dst + units * 16), tail);
+                       (unsigned short*)((char*)dst + units * 16), tail, g_copy_streaming_stores);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }

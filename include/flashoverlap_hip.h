@@ -134,7 +134,11 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host);
  *                  instead (L2 write-back first), with the tile stores as
  *                  "store_mode" says.
  *   "store_mode"   with release_mode 0 only.  1 (default): write-through tile
- *                  stores; 0: cached tile stores. */
+ *                  stores; 0: cached tile stores.
+ *   "copy_streaming_stores"  0 (default): the consumer copies (fo_consume,
+ *                  fo_wait_consume) store with ordinary stores, so their
+ *                  destination may stay in the memory-side cache for its
+ *                  reader; 1: non-temporal stores. */
 int fo_tune(const char* key, int value);
 
 /* ---- counting / wait -------------------------------------------------- */
