@@ -229,8 +229,23 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     const int cp_row = lane >> 3;
     const int cp_off0 = (cp_row * K + ((lane & 7) ^ swz(cp_row)) * 8) * 2;       // even slabs
     const int cp_off1 = (cp_row * K + ((lane & 7) ^ swz(cp_row + 8)) * 8) * 2;   // odd slabs
-    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, 0xffffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, 0xffffffff, 0x00020000);
+    // K need not be a multiple of the panel depth.  In the last, partial panel the
+    // lanes whose k-chunk lies beyond K take a per-lane offset outside the buffer's
+    // range instead: the hardware then fetches nothing for them and writes zeros to
+    // their LDS bytes, so the panel is zero-padded and the main loop needs no k
+    // mask.  The range (2 GiB, checked against the operand sizes on the host) only
+    // has to separate that one offset from the real ones.
+    const int k_rest = K % kBK;
+    constexpr int kOutOfRange = (int)0x80000000u;
+    int tail_off0 = cp_off0, tail_off1 = cp_off1;
+    if (k_rest) {
+        if (((lane & 7) ^ swz(cp_row)) * 8 >= k_rest) tail_off0 = kOutOfRange;
+        if (((lane & 7) ^ swz(cp_row + 8)) * 8 >= k_rest) tail_off1 = kOutOfRange;
+    }
+    int vo0 = cp_off0, vo1 = cp_off1;   // the offsets in use: the tail pair for the last panel
+    const int range = k_rest ? kOutOfRange : (int)0xffffffffu;
+    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, range, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, range, 0x00020000);
     const unsigned baseA = (unsigned)(mt.m * MT + wave * (LOADS * 8)) * (unsigned)K * 2u;
     const unsigned baseB = (unsigned)(mt.n * MT + wave * (LOADS * 8)) * (unsigned)K * 2u;
     const unsigned slab_bytes = 8u * (unsigned)K * 2u;    // bytes between consecutive slabs
@@ -246,7 +261,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         const unsigned koff = (unsigned)kt * (kBK * 2);
 #pragma unroll
         for (int j = H * (LOADS / 2); j < (H + 1) * (LOADS / 2); ++j) {
-            const int voff = (j & 1) ? cp_off1 : cp_off0;   // LOADS*8 is a multiple of 16: slab parity = j parity
+            const int voff = (j & 1) ? vo1 : vo0;   // LOADS*8 is a multiple of 16: slab parity = j parity
             if constexpr (ISB)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, voff,
                                                          (int)(baseB + j * slab_bytes + koff), 0, 0);
@@ -307,7 +322,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    const int NP = K / kBK;   // panels
+    const int NP = (K + kBK - 1) / kBK;   // panels, the last one possibly partial
     // One k-step on panel kt, whose A and B units sit in slots sa and sb; the
     // units of panel kt+1 are in na and nb (landed or landing), sp is the free
     // slot.  On entry the fragments of the first quarter are in registers.  All
@@ -323,7 +338,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         constexpr int j = decltype(j_c)::value;
         unsigned char* dst = smem + slot + lds_cp;
         const unsigned koff = (unsigned)kt * (kBK * 2);
-        const int voff = (j & 1) ? cp_off1 : cp_off0;
+        const int voff = (j & 1) ? vo1 : vo0;
         if constexpr (ISB)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, voff,
                                                      (int)(baseB + j * slab_bytes + koff), 0, 0);
@@ -399,11 +414,19 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     };
 
     // Prologue: panels 0 and 1 go out; wait for panel 0.
+    auto last_panel_next = [&](bool is_last) {   // called before the copies of a panel are issued
+        if (is_last) {
+            vo0 = tail_off0;
+            vo1 = tail_off1;
+        }
+    };
+    last_panel_next(NP == 1);
     issue_unit(0, 0 * PANEL, unit_a, first_half);
     issue_unit(0, 0 * PANEL, unit_a, second_half);
     issue_unit(0, 1 * PANEL, unit_b, first_half);
     issue_unit(0, 1 * PANEL, unit_b, second_half);
     if (NP > 1) {
+        last_panel_next(NP == 2);
         issue_unit(1, 2 * PANEL, unit_a, first_half);
         issue_unit(1, 2 * PANEL, unit_a, second_half);
         issue_unit(1, 3 * PANEL, unit_b, first_half);
@@ -426,6 +449,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         sa = na; sb = nb; na = sp; nb = a0; sp = b0;
     };
     for (; kt < NP - 2; ++kt) {
+        last_panel_next(kt + 3 == NP);   // this k-step copies panel kt + 2
         kstep(kt, sa, sb, na, nb, sp, std::true_type{}, std::true_type{});
         rotate();
     }
@@ -569,11 +593,13 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
     if (!A || !B || !D) return fail(FO_ERR_ARG, "fo_gemm: null operand");
     if (M <= 0 || N <= 0 || K <= 0) return fail(FO_ERR_SHAPE, "fo_gemm: empty problem %dx%dx%d", M, N, K);
     if (M % BM || N % BN) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d not multiples of the %dx%d tile", M, N, BM, BN);
-    if (K % kBK) return fail(FO_ERR_SHAPE, "fo_gemm: K=%d not a multiple of %d", K, kBK);
+    if (K % 8) return fail(FO_ERR_SHAPE, "fo_gemm: K=%d not a multiple of 8 (operand rows must be 16-byte aligned)", K);
     if ((long long)M * N >= (1LL << 31)) return fail(FO_ERR_LIMIT, "fo_gemm: M*N=%lld needs 64-bit tile offsets", (long long)M * N);
     if ((long long)M * K >= (1LL << 31) || (long long)N * K >= (1LL << 31))
         return fail(FO_ERR_LIMIT, "fo_gemm: an operand of %lld elements exceeds the 4 GiB a buffer descriptor addresses",
                     (long long)(M > N ? M : N) * K);
+    if (K % kBK && ((long long)M * K >= (1LL << 30) || (long long)N * K >= (1LL << 30)))
+        return fail(FO_ERR_LIMIT, "fo_gemm: K=%d is not a multiple of %d and an operand exceeds the 2 GiB this case addresses", K, kBK);
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)D) & 15) return fail(FO_ERR_ARG, "fo_gemm: operands must be 16-byte aligned");
     const int macro = choose_macro_tile(BM, BN, M, N);
     if (!macro) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d unsupported for tile %dx%d (need multiples of 256, or 128 with the 128x128 tile)", M, N, BM, BN);

@@ -64,7 +64,8 @@ int fo_device_info(int* cu_count, int* clock_khz, int* xcd_count);
 /* D[M,N] = A[M,K] . B[N,K]^T, fp32 accumulate, natural row-major D.
  * Replaces gemm_func_table[Algo] / mutlass_gemm<TM,TN,TK>
  * (src/tiling/gemm_dispatcher.h:16-20, src/gemm/gemm.cu:29-113).
- * Requires M % BM == 0, N % BN == 0, K % 64 == 0, 16-byte aligned pointers. */
+ * Requires M % BM == 0, N % BN == 0, K % 8 == 0 (a K that is not a multiple of 64
+ * is zero-padded inside the kernel; the operands must then be below 2 GiB each), 16-byte aligned pointers. */
 int fo_gemm(int dtype, int algo, int M, int N, int K,
             const void* A, const void* B, void* D, void* stream);
 

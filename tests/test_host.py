@@ -47,7 +47,7 @@ def test_argument_errors_return_codes_not_exits(fo_lib):
     # shape / argument validation happens before any device call
     rc = fo_lib.fo_gemm(capi.FO_F16, 1, 100, 128, 64, 16, 16, 16, None)
     assert rc == capi.FO_ERR_SHAPE and b"multiples" in fo_lib.fo_last_error()
-    assert fo_lib.fo_gemm(capi.FO_F16, 1, 128, 128, 40, 16, 16, 16, None) == capi.FO_ERR_SHAPE
+    assert fo_lib.fo_gemm(capi.FO_F16, 1, 128, 128, 36, 16, 16, 16, None) == capi.FO_ERR_SHAPE
     assert fo_lib.fo_gemm(7, 1, 128, 128, 64, 16, 16, 16, None) == capi.FO_ERR_ARG
     assert fo_lib.fo_gemm(capi.FO_F16, 9, 128, 128, 64, 16, 16, 16, None) == capi.FO_ERR_ARG
     assert fo_lib.fo_gemm(capi.FO_F16, 1, 128, 128, 64, None, 16, 16, None) == capi.FO_ERR_ARG

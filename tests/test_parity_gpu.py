@@ -135,7 +135,10 @@ def _timeouts(L):
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K,algo", [(128, 128, 64, 1), (256, 256, 64, 0), (256, 512, 192, 3), (512, 256, 128, 5),
-                                        (384, 640, 320, 1), (1024, 1024, 1024, 1), (2048, 4096, 256, 1)])
+                                        (384, 640, 320, 1), (1024, 1024, 1024, 1), (2048, 4096, 256, 1),
+                                        # K that is not a multiple of the 64-deep panel: a zero-padded last panel
+                                        (128, 128, 8, 1), (256, 256, 72, 0), (256, 512, 200, 3), (512, 256, 120, 5),
+                                        (384, 640, 328, 1), (1024, 1024, 1000, 1)])
 def test_gemm_bit_exact_on_integer_inputs(L, dev, dt, M, N, K, algo):
     _say("gemm integer", dt, M, N, K, algo)
     p = Path(L, dev, dt, M, N, K, algo, integer_inputs=True)
@@ -145,9 +148,10 @@ def test_gemm_bit_exact_on_integer_inputs(L, dev, dt, M, N, K, algo):
     assert torch.equal(got.cpu(), want)
 
 
+@pytest.mark.parametrize("K", [2048, 2040])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
-def test_gemm_random_within_tolerance(L, dev, dt):
-    M, N, K = 1024, 768, 2048
+def test_gemm_random_within_tolerance(L, dev, dt, K):
+    M, N = 1024, 768
     _say("gemm random", dt, M, N, K)
     p = Path(L, dev, dt, M, N, K, 1, seed=3)
     got = p.gemm_plain().cpu()
@@ -162,7 +166,7 @@ def test_gemm_random_within_tolerance(L, dev, dt):
 
 def test_gemm_rejects_unsupported_shapes(L, dev):
     a = torch.zeros(384, 384, dtype=torch.float16, device=dev)  # large enough for every call below
-    assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 48, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
+    assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 44, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
     assert L.fo_gemm(capi.FO_F16, 3, 384, 384, 64, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
 
 
@@ -171,6 +175,7 @@ def test_gemm_rejects_unsupported_shapes(L, dev):
 @pytest.mark.parametrize("dt,M,N,K,algo,w", [
     (torch.float16, 1024, 1024, 1024, 1, 4),      # benchmark configuration 1: 64 tiles, 16 groups of 4 (> TN = 8 counters)
     (torch.bfloat16, 512, 768, 128, 1, 5),        # ragged last group
+    (torch.bfloat16, 512, 768, 136, 1, 5),        # the same with a partial last k panel
     (torch.float16, 1024, 2048, 64, 3, 3),        # 128x256 layout tile
     (torch.bfloat16, 2048, 1024, 64, 5, 7),       # 256x128 layout tile
     (torch.float16, 2048, 2048, 64, 1, 1),        # one tile per group: 256 counters
