@@ -105,9 +105,12 @@ def main() -> int:
     ap.add_argument("--consumer-blocks", type=int, default=0,
                     help="workgroups of the persistent consumer (0 = one per CU, which is also the maximum)")
     ap.add_argument("--consumer", default="auto", choices=["auto", "per_group", "persistent"])
-    ap.add_argument("--last-group", default="main", choices=["main", "comm"],
-                    help="stream that releases the last group (per-group consumer): the GEMM's own (default, what "
-                         "OverlapImpl does) or the second stream like every other group")
+    ap.add_argument("--last-group", default="settle_then_join", choices=["main", "comm", "settle", "settle_then_join"],
+                    help="how the last group is released (per-group consumer): settle_then_join (default, what "
+                         "OverlapImpl does): on the GEMM's own stream by one launch that settles the counter and copies, "
+                         "the earlier groups joined behind it; settle: the same with the join in front; main: wait "
+                         "kernel + copy on the GEMM's stream behind the join; comm: on the second stream like every "
+                         "other group, as the reference does")
     ap.add_argument("--no-overlap", action="store_true",
                     help="order the consumer behind the GEMM in the timed step (needed under counter collection, "
                          "which runs one kernel at a time)")
@@ -209,20 +212,26 @@ def main() -> int:
         acc = 0
         for gi, n in enumerate(g.cseg):
             stream = comm
-            if gi == g.G - 1 and a.last_group == "main":
-                # the last group completes with the GEMM: release it on the GEMM's stream, behind a join
-                # (of the groups before it) that was satisfied long ago
-                if g.G > 1:
+            last_on_main = gi == g.G - 1 and a.last_group != "comm"
+            if last_on_main:
+                # the last group completes with the GEMM: release it on the GEMM's stream
+                if g.G > 1 and a.last_group != "settle_then_join":
                     capi.check(L.fo_stream_join(comm, main_stream))
                 stream = main_stream
-            capi.check(L.fo_wait(n, g.MM.data_ptr() + 4 * gi, stream))
+            settle = last_on_main and a.last_group != "main"
+            if not settle:
+                capi.check(L.fo_wait(n, g.MM.data_ptr() + 4 * gi, stream))
             elems = n * BM * BN
             part = elems // ws
             for k in range(ws):  # ws > 1: slice k of the group goes to rank k's receive buffer
-                capi.check(L.fo_consume(Cp.data_ptr() + 2 * (acc + k * part),
-                                        staging.data_ptr() + 2 * (k * (M * N // ws) + acc // ws), 2 * part, stream))
+                src = Cp.data_ptr() + 2 * (acc + k * part)
+                dst = staging.data_ptr() + 2 * (k * (M * N // ws) + acc // ws)
+                if settle and k == 0:
+                    capi.check(L.fo_settle_consume(n, g.MM.data_ptr() + 4 * gi, src, dst, 2 * part, stream))
+                else:
+                    capi.check(L.fo_consume(src, dst, 2 * part, stream))
             acc += elems
-        if a.last_group != "main":
+        if a.last_group == "comm" or (a.last_group == "settle_then_join" and g.G > 1):
             capi.check(L.fo_stream_join(comm, main_stream))
 
     def norm(i=0):
@@ -277,7 +286,10 @@ def main() -> int:
 
     def consumer_name(g):
         return ("one wait kernel + one copy launch per group"
-                + (", the last group on the GEMM's stream" if a.last_group == "main" and g.G > 1 else "")
+                + {"comm": "", "main": ", the last group on the GEMM's stream",
+                   "settle": ", the last group settled and copied by one launch on the GEMM's stream",
+                   "settle_then_join": ", the last group settled and copied by one launch on the GEMM's stream"}[
+                       a.last_group]
                 if g.per_group else
                 f"persistent wait+consume, {a.consumer_blocks} workgroups")
 

@@ -35,6 +35,7 @@ SIGNATURES = {
     "fo_set_wait_timeout_ms": (_i, [_i]),
     "fo_wait_timeouts": (_i, [_ip, _i]),
     "fo_consume": (_i, [_vp, _vp, _sz, _vp]),
+    "fo_settle_consume": (_i, [_i, _vp, _vp, _vp, _sz, _vp]),
     "fo_reorder_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "fo_reorder_rmsnorm_batched": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "fo_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _f, _vp]),

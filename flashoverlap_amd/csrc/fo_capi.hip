@@ -114,6 +114,11 @@ int fo_consume(const void* src, void* dst, size_t bytes, void* stream) {
     return launch_consume(src, dst, bytes, (hipStream_t)stream);
 }
 
+int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t bytes, void* stream) {
+    if (!addr) return fail(FO_ERR_ARG, "fo_settle_consume: null counter address");
+    return launch_consume(src, dst, bytes, (hipStream_t)stream, that, addr);
+}
+
 int fo_reorder_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
                        int rldn, const int* RA, float eps, void* stream) {
     if (!RA) return fail(FO_ERR_ARG, "fo_reorder_rmsnorm: null RA");

@@ -190,7 +190,17 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
 
 __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                                long long units, const unsigned short* src_tail,
-                                                               unsigned short* dst_tail, int tail, int streaming_stores) {
+                                                               unsigned short* dst_tail, int tail, int streaming_stores,
+                                                               int that, int* addr) {
+    // Settling a counter whose producer ran earlier on this stream takes no
+    // waiting: it holds its final value.  The right value is cleared like
+    // wait_kernel does; a wrong one is left and counted like an expired wait.
+    if (addr && blockIdx.x == 0 && threadIdx.x == 0) {
+        if (__hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == that)
+            __hip_atomic_store(addr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+            atomicAdd(&g_wait_timeouts, 1);
+    }
     team_copy<false, kCopyThreads>(src, dst, units, blockIdx.x, gridDim.x, threadIdx.x, streaming_stores);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
@@ -309,8 +319,8 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
     return FO_OK;
 }
 
-int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream) {
-    if (bytes == 0) return FO_OK;
+int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream, int that, int* addr) {
+    if (bytes == 0 && !addr) return FO_OK;
     if (!src || !dst) return fail(FO_ERR_ARG, "fo_consume: null buffer");
     if (bytes & 1) return fail(FO_ERR_ARG, "fo_consume: %zu bytes is not a whole number of 16-bit elements", bytes);
     if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_consume: buffers must be 16-byte aligned");
@@ -322,7 +332,7 @@ int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream)
     if (blocks == 0) blocks = 1;
     hipLaunchKernelGGL(consume_kernel, dim3((unsigned)blocks), dim3(kCopyThreads), 0, stream, (const uint4*)src,
                        (uint4*)dst, (long long)units, (const unsigned short*)((const char*)src + units * 16),
-                       (unsigned short*)((char*)dst + units * 16), tail, g_copy_streaming_stores);
+                       (unsigned short*)((char*)dst + units * 16), tail, g_copy_streaming_stores, that, addr);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }

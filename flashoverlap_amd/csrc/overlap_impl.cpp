@@ -166,23 +166,28 @@ void OverlapImpl::consume_groups(const at::Tensor& C, void* dst, int64_t tile_el
     int64_t acc = 0;
     for (int g = 0; g < G; ++g) {
         // The last group completes with the GEMM, so nothing is left for it to overlap with:
-        // it is released on the GEMM's own stream, behind the join of the groups before it.
-        // That join has been satisfied long before the stream reaches it, whereas a join
-        // behind the last group would put a fresh cross-stream dependency (10-20 us on this
-        // platform) between the last copy and the caller's next kernel.
-        void* stream = comm_stream_;
-        if (g == G - 1) {
-            if (G > 1) FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
-            stream = gemm_stream_;
-        }
+        // it is released on the GEMM's own stream, where stream order stands in for the wait
+        // kernel (the counter is settled by the copy launch itself), and the groups before it,
+        // finished long ago on the communication stream, are joined behind it.  A last group
+        // on the communication stream would instead put a fresh cross-stream dependency
+        // (10-20 us on this platform) between its copy and the caller's next kernel.
+        const bool last = g == G - 1;
+        void* stream = last ? gemm_stream_ : comm_stream_;
         const int64_t comm = tile_elems * cseg[g];
-        FO_CALL(fo_wait(cseg[g], MM.data_ptr<int>() + g, stream));
+        if (!last) FO_CALL(fo_wait(cseg[g], MM.data_ptr<int>() + g, stream));
         const int64_t part = comm / nslices;
-        for (int k = 0; k < slice_count; ++k)
-            FO_CALL(fo_consume(src + (acc + (slice_first + k) * part) * esz,
-                               (char*)dst + (k * slice_stride + acc / nslices) * esz, part * esz, stream));
+        for (int k = 0; k < slice_count; ++k) {
+            const void* from = src + (acc + (slice_first + k) * part) * esz;
+            void* to = (char*)dst + (k * slice_stride + acc / nslices) * esz;
+            if (last && k == 0)
+                FO_CALL(fo_settle_consume(cseg[g], MM.data_ptr<int>() + g, from, to, part * esz, stream));
+            else
+                FO_CALL(fo_consume(from, to, part * esz, stream));
+        }
         acc += comm;
     }
+    // The caller's stream continues only after every group is consumed (src/overlap_impl.cu:267-270).
+    if (G > 1) FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
 }
 
 void OverlapImpl::GemmAllReduceOverlap(at::Tensor A, at::Tensor B, at::Tensor C, at::Tensor MM, at::Tensor RA,

@@ -190,6 +190,16 @@ int fo_wait_timeouts(int* count, int reset);
  * group (call sites src/overlap_impl.cu:263, 319-320). */
 int fo_consume(const void* src, void* dst, size_t bytes, void* stream);
 
+/* fo_wait + fo_consume in one launch, for a group whose producing GEMM was
+ * enqueued earlier on the same `stream`: stream order has already made the
+ * counter final, so there is nothing to poll.  *addr == that is cleared to 0 as
+ * fo_wait does; any other value is left in place and counted as an expired wait
+ * (fo_wait_timeouts).  The copy is made either way, as it would be behind an
+ * expired fo_wait.  Used for the last group of a call, which completes together
+ * with the GEMM (the reference waits for it on the communication stream,
+ * src/overlap_impl.cu:257-265, and then joins the streams). */
+int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t bytes, void* stream);
+
 /* ---- RMSNorm ---------------------------------------------------------- */
 
 /* out[b,:] = rmsnorm(gather(x)[b,:]) * gamma, gather as in the layout header.

@@ -365,6 +365,27 @@ def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
         capi.check(L.fo_set_wait_timeout_ms(5000))
 
 
+def test_settle_consume_clears_the_right_count_and_reports_a_wrong_one(L, dev, comm_stream):
+    """The last group's launch: behind its producer on one stream the counter is final, so the
+    launch checks it instead of waiting (same outcome as src/wait.cuh:5-9 on the right count)."""
+    mm = torch.tensor([7, 9, 0], dtype=torch.int32, device=dev)
+    src = torch.randint(-30000, 30000, (40000,), dtype=torch.int16, device=dev)
+    dst = torch.zeros_like(src)
+    capi.check(L.fo_settle_consume(7, mm.data_ptr(), src.data_ptr(), dst.data_ptr(), 2 * 40000, comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 0 and torch.equal(dst, src)
+    # a wrong count stays where it is and is counted, at once (no polling); the copy is still made
+    dst.zero_()
+    capi.check(L.fo_settle_consume(8, mm.data_ptr() + 4, src.data_ptr(), dst.data_ptr(), 2 * 40000, comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 1 and torch.equal(dst, src)
+    # an empty group still settles its counter
+    capi.check(L.fo_settle_consume(0, mm.data_ptr() + 8, src.data_ptr(), dst.data_ptr(), 0, comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 0
+    assert L.fo_settle_consume(0, None, src.data_ptr(), dst.data_ptr(), 16, comm_stream) == capi.FO_ERR_ARG
+
+
 def test_consume_copies_exactly_the_bytes(L, dev):
     src = torch.randint(-30000, 30000, (100003,), dtype=torch.int16, device=dev)
     for off, n in ((0, 100003), (8, 77), (16, 8), (24, 4099)):
