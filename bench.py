@@ -244,6 +244,10 @@ def main() -> int:
                                             1, RA.data_ptr(), eps, main_stream))
 
     def step(g, overlap=True, ev=None):
+        if overlap and (g.G > 1 or not g.per_group):
+            # like OverlapImpl: the second stream's part of the step is ordered behind what the main stream
+            # held before the GEMM (a fork, so that the step is a fork/join pattern on the main stream)
+            capi.check(L.fo_stream_join(main_stream, comm))
         if ev:
             tm.record(ev[0])
         gemm_signal(g)

@@ -141,6 +141,16 @@ void OverlapImpl::Gemm(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo) {
     FO_CALL(fo_gemm(s.dtype, (int)Algo, s.M, s.N, s.K, A.data_ptr(), B.data_ptr(), C.data_ptr(), gemm_stream_));
 }
 
+// Called before the GEMM is enqueued: the communication stream's part of this call is
+// ordered behind what the GEMM's stream held so far (not behind the GEMM itself).  The wait
+// kernels lose nothing by it (their GEMM cannot start earlier either), and it makes the call
+// a fork/join pattern on the caller's stream, which is what stream capture into a graph needs
+// to follow the work onto the second stream.
+void OverlapImpl::fork_comm_stream(int G) {
+    const bool persistent = consumer_mode_ == 2 || (consumer_mode_ == 0 && G > 32);
+    if (persistent || G > 1) FO_CALL(fo_stream_join(gemm_stream_, comm_stream_));
+}
+
 // Per-group release: either the reference's host loop (one wait kernel and one
 // consumer launch per group, src/overlap_impl.cu:257-265 / 312-323) or one
 // persistent kernel that does the same walk on the device.  On return the GEMM
@@ -201,6 +211,7 @@ void OverlapImpl::GemmAllReduceOverlap(at::Tensor A, at::Tensor B, at::Tensor C,
     c10::DeviceGuard guard(A.device());
     at::Tensor& staging = staging_like(C);
     const int* table = group_table_for(cSEG_CPU, cSEG_GPU, g.T);
+    fork_comm_stream(g.G);
     FO_CALL(fo_gemm_signal(s.dtype, (int)Algo, s.M, s.N, s.K, (int)rLDN, cSEG_GPU.data_ptr<int>(), g.G, table,
                            A.data_ptr(), B.data_ptr(), C.data_ptr(), MM.data_ptr<int>(), RA.data_ptr<int>(),
                            if_monitor ? 1 : 0, gemm_stream_));
@@ -225,6 +236,7 @@ void OverlapImpl::GemmReduceScatterOverlap(at::Tensor A, at::Tensor B, at::Tenso
                 " elements, got ", D.numel());
     c10::DeviceGuard guard(A.device());
     const int* table = group_table_for(cSEG_CPU, cSEG_GPU, g.T);
+    fork_comm_stream(g.G);
     FO_CALL(fo_gemm_scatter(s.dtype, (int)Algo, s.M, s.N, s.K, (int)rLDN, cSEG_GPU.data_ptr<int>(), g.G, table,
                             A.data_ptr(), B.data_ptr(), C.data_ptr(), MM.data_ptr<int>(), RA.data_ptr<int>(),
                             RE.data_ptr<int>(), if_monitor ? 1 : 0, gemm_stream_));

@@ -88,6 +88,7 @@ class OverlapImpl : public torch::CustomClassHolder {
     void require_overlap() const;
     at::Tensor& staging_like(const at::Tensor& C);
     const int* group_table_for(const at::Tensor& cseg_cpu, const at::Tensor& cseg_gpu, int T);
+    void fork_comm_stream(int G);
     void consume_groups(const at::Tensor& C, void* dst, int64_t tile_elems, const at::Tensor& cseg_cpu,
                         const at::Tensor& cseg_gpu, at::Tensor& MM, int nslices, int64_t slice_stride);
     void bulk_consume(const void* src, void* dst, size_t bytes);
