@@ -90,6 +90,22 @@ struct Mma<__bf16> {
     }
 };
 
+// The MFMAs above are opaque to the compiler: it does not know that their
+// results become readable only some cycles after issue, and it inserts no wait
+// states between one of them and an instruction that reads its accumulator.  So
+// the accumulators are kept in the matrix-core register file (constraint "a")
+// from the first MFMA to the epilogue, where they are read by this statement
+// behind an explicit settle() — the compiler is then never asked to move an
+// accumulator on its own (a copy it places right behind an MFMA reads the value
+// from before that MFMA).
+static __device__ __forceinline__ float acc_read(const float& a) {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+// More wait states than the longest MFMA needs before its result can be read.
+static __device__ __forceinline__ void settle_mfma() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+
 constexpr int kBK = 64;             // k-elements per LDS buffer
 constexpr int kRowBytes = kBK * 2;  // one panel row in LDS: 128 bytes = 8 chunks of 16
 
@@ -182,6 +198,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 
     const TileCoord mt = raster_map(blockIdx.x, p.GM, p.GN);
     const int K = p.K;
+    // M and N are multiples of the layout tile, not necessarily of the macro
+    // tile: the last row or column of macro tiles may be half inside.  Such a
+    // workgroup runs the full main loop (the waves of the outer half re-read the
+    // panel rows of the inner half, so nothing outside the operands is touched)
+    // and only the quadrants inside are stored and signalled.
+    const int valid_m = min(MT, p.M - mt.m * MT), valid_n = min(MT, p.N - mt.n * MT);   // MT or MT / 2
+    const bool live = wm * WT < valid_m && wn * WT < valid_n;                          // this wave's quadrant
 
     // ---- where this wavefront's quadrant goes -------------------------------
     // row0/col0/ld describe the destination of quadrant element (0,0) in a
@@ -197,14 +220,15 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         const int tiles_m = MT / p.BM;
         const int qm = wm * WT, qn = wn * WT;         // quadrant origin in the macro tile
         const int t = (mt.m * tiles_m + qm / p.BM) * p.TN + mt.n * tiles_n + qn / p.BN;
-        const int s = __builtin_amdgcn_readfirstlane(p.RA[t]);
+        const int s = live ? __builtin_amdgcn_readfirstlane(p.RA[t]) : 0;
         row0 = (s / p.rLDN) * p.BM + qm % p.BM;
         col0 = (s % p.rLDN) * p.BN + qn % p.BN;
         ld = p.rLDN * p.BN;
         // The lanes that will signal look up their slot and group now, so the
         // two dependent loads are hidden behind the main loop.
         const int ntile = tiles_m * tiles_n;
-        if (tid < ntile) {
+        sig_group = -1;   // lanes without a layout tile (or with one outside the matrix) stay out of the signal
+        if (tid < ntile && (tid / tiles_n) * p.BM < valid_m && (tid % tiles_n) * p.BN < valid_n) {
             const int ts = (mt.m * tiles_m + tid / tiles_n) * p.TN + mt.n * tiles_n + tid % tiles_n;
             sig_slot = p.RA[ts];
             sig_group = p.gtable ? p.gtable[sig_slot] : scan_group(p.cseg, sig_slot);
@@ -246,8 +270,8 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     const int range = k_rest ? kOutOfRange : (int)0xffffffffu;
     const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, range, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, range, 0x00020000);
-    const unsigned baseA = (unsigned)(mt.m * MT + wave * (LOADS * 8)) * (unsigned)K * 2u;
-    const unsigned baseB = (unsigned)(mt.n * MT + wave * (LOADS * 8)) * (unsigned)K * 2u;
+    const unsigned baseA = (unsigned)(mt.m * MT + ((wave * (LOADS * 8)) & (valid_m - 1))) * (unsigned)K * 2u;
+    const unsigned baseB = (unsigned)(mt.n * MT + ((wave * (LOADS * 8)) & (valid_n - 1))) * (unsigned)K * 2u;
     const unsigned slab_bytes = 8u * (unsigned)K * 2u;    // bytes between consecutive slabs
     const int lds_cp = wave * (LOADS * 1024);             // this wave's first slab in a panel
 
@@ -463,6 +487,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     // ---- epilogue: registers -> LDS strip -> global -------------------------------
     // acc[i][j][r] is element m = 16i + l%16, n = 16j + 4(l/16) + r (fr_g = l/16).
     __builtin_amdgcn_s_setprio(0);
+    settle_mfma();
     __syncthreads();  // every wave is done with the panel buffers
     constexpr int PITCH = WT * 2 + 16;                  // strip row pitch in bytes
     constexpr int ROWCH = WT / 8;                       // 16-byte chunks per strip row
@@ -478,7 +503,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
             for (int j = 0; j < NB; ++j) {
                 out4 o;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = (T)acc[2 * i + ii][j][r];
+                for (int r = 0; r < 4; ++r) o[r] = (T)acc_read(acc[2 * i + ii][j][r]);
                 *(out4*)(ep + (16 * ii + fr_row) * PITCH + (16 * j + 4 * fr_g) * 2) = o;
             }
 #pragma unroll
@@ -492,6 +517,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
                 row = __shfl((WT > 64 && i >= 2) ? re_hi : re_lo, q_row & 63, 64);
             }
             const size_t off = (size_t)row * ld + col0 + cc * 8;
+            if (!live) continue;   // a quadrant outside the matrix goes through the motions and stores nothing
             if constexpr (STORE == 1)
                 __builtin_amdgcn_raw_buffer_store_b128(v, drsrc, (int)(off * 2), 0, 16);  // sc1: write-through
             else
@@ -517,13 +543,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int o = 0; o < 4; ++o) {
                 const int g = __shfl(sig_group, o, 64);
-                if (o < ntile && g == sig_group) {
+                if (o < ntile && g == sig_group && g >= 0) {
                     ++same;
                     if (o < tid) ++earlier;
                 }
             }
         }
-        if (tid < ntile && (p.monitor || earlier == 0)) {
+        if (tid < ntile && sig_group >= 0 && (p.monitor || earlier == 0)) {
             const int add = p.monitor ? 1 : same;
             if constexpr (REL == 1)  // the stores already went through to memory
                 __hip_atomic_fetch_add(p.MM + sig_group, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -572,16 +598,16 @@ static int launch_mt(int mode, const GemmParams& p, hipStream_t stream) {
 }
 
 int choose_macro_tile(int BM, int BN, int M, int N) {
-    const bool ok256 = (M % 256 == 0) && (N % 256 == 0) && (256 % BM == 0) && (256 % BN == 0);
-    const bool ok128 = (BM == 128 && BN == 128) && (M % 128 == 0) && (N % 128 == 0);
-    if (ok256 && ok128) {
+    if (M % BM || N % BN) return 0;
+    // Every layout tile (128 or 256 on a side) divides the 256x256 macro tile; a matrix edge
+    // that is an odd multiple of 128 is covered by half a macro tile.
+    const bool ok128 = BM == 128 && BN == 128;
+    if (ok128) {
         // Small problems: prefer the tile that puts work on more CUs.
-        const int wg256 = (M / 256) * (N / 256);
-        return wg256 >= 128 ? 256 : 128;
+        const int wg256 = ((M + 255) / 256) * ((N + 255) / 256);
+        if (wg256 < 128) return 128;
     }
-    if (ok256) return 256;
-    if (ok128) return 128;
-    return 0;
+    return 256;
 }
 
 int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg, int G,
@@ -602,12 +628,12 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
         return fail(FO_ERR_LIMIT, "fo_gemm: K=%d is not a multiple of %d and an operand exceeds the 2 GiB this case addresses", K, kBK);
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)D) & 15) return fail(FO_ERR_ARG, "fo_gemm: operands must be 16-byte aligned");
     const int macro = choose_macro_tile(BM, BN, M, N);
-    if (!macro) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d unsupported for tile %dx%d (need multiples of 256, or 128 with the 128x128 tile)", M, N, BM, BN);
+    if (!macro) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d not multiples of the %dx%d tile", M, N, BM, BN);
 
     GemmParams p{};
     p.A = A; p.B = B; p.D = D;
     p.M = M; p.N = N; p.K = K;
-    p.GM = M / macro; p.GN = N / macro;
+    p.GM = (M + macro - 1) / macro; p.GN = (N + macro - 1) / macro;
     p.BM = BM; p.BN = BN; p.TN = N / BN;
     p.rLDN = rLDN;
     p.RA = RA; p.RE = RE; p.cseg = cseg; p.G = G; p.gtable = gtable; p.MM = MM; p.monitor = monitor;
@@ -631,13 +657,16 @@ int raster_hint(int algo, int M, int N, int* hint) {
     if (M <= 0 || N <= 0 || M % BM || N % BN) return fail(FO_ERR_SHAPE, "fo_raster_hint: M=%d N=%d vs tile %dx%d", M, N, BM, BN);
     const int macro = choose_macro_tile(BM, BN, M, N);
     if (!macro) return fail(FO_ERR_SHAPE, "fo_raster_hint: M=%d N=%d unsupported for tile %dx%d", M, N, BM, BN);
-    const int GM = M / macro, GN = N / macro, TN = N / BN;
+    const int GM = (M + macro - 1) / macro, GN = (N + macro - 1) / macro, TM = M / BM, TN = N / BN;
     const int tiles_m = macro / BM, tiles_n = macro / BN;
     int k = 0;
     for (int pid = 0; pid < GM * GN; ++pid) {
         const TileCoord c = raster_map(pid, GM, GN);
         for (int i = 0; i < tiles_m; ++i)
-            for (int j = 0; j < tiles_n; ++j) hint[k++] = (c.m * tiles_m + i) * TN + c.n * tiles_n + j;
+            for (int j = 0; j < tiles_n; ++j) {
+                const int tm = c.m * tiles_m + i, tn = c.n * tiles_n + j;
+                if (tm < TM && tn < TN) hint[k++] = tm * TN + tn;   // half macro tiles at the matrix edge
+            }
     }
     return FO_OK;
 }

@@ -1,0 +1,88 @@
+"""Build-time checks on the code the compiler makes of the GEMM kernel (no GPU needed).
+
+The kernel issues its MFMAs from inline assembly, which the compiler treats as
+opaque: it neither knows their latency nor inserts the wait states the hardware
+needs between an MFMA and a read of its accumulator.  The source therefore keeps
+the accumulators in the matrix-core register file and reads them itself behind an
+explicit delay.  These checks make a build fail if the compiler ever places an
+accumulator access of its own close behind an MFMA, and keep the register budget
+that lets the consumer's wavefronts run beside the GEMM's.
+"""
+import os
+import re
+import subprocess
+
+import pytest
+
+from flashoverlap_amd import build
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+MIN_WAIT_STATES = 16   # the longest MFMA of this family needs fewer before its result may be read
+
+
+@pytest.fixture(scope="module")
+def gemm_asm(tmp_path_factory):
+    hipcc = os.path.join(build.ROCM, "bin", "hipcc")
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    out = tmp_path_factory.mktemp("asm") / "fo_gemm.s"
+    flags = [f for f in build.HIPCC_FLAGS if f != "-fPIC"]
+    cmd = [hipcc, *flags, "--cuda-device-only", "-S", os.path.join(build.CSRC, "fo_gemm.hip"), "-o", str(out)]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=600)
+    return out.read_text()
+
+
+def _kernels(text):
+    """name -> (instruction lines, metadata dict) for every gemm_kernel instantiation."""
+    bodies, name = {}, None
+    for line in text.splitlines():
+        m = re.match(r"^(_ZN2fo11gemm_kernel\S+):", line)
+        if m:
+            name = m.group(1)
+            bodies[name] = []
+            continue
+        if name:
+            if line.startswith(".Lfunc_end"):
+                name = None
+                continue
+            code = line.split(";")[0].strip()
+            if code:
+                bodies[name].append(code)
+    meta = {}
+    for m in re.finditer(r"\.name:\s+(_ZN2fo11gemm_kernel\S+)\n(?:.*\n)*?\s+\.vgpr_count:\s+(\d+)\n\s+\.vgpr_spill_count:\s+(\d+)",
+                         text):
+        meta[m.group(1)] = {"vgpr": int(m.group(2)), "spill": int(m.group(3))}
+    return bodies, meta
+
+
+AGPR = re.compile(r"\ba(\d+|\[\d+:\d+\])")
+
+
+def test_no_accumulator_access_close_behind_an_mfma(gemm_asm):
+    bodies, _ = _kernels(gemm_asm)
+    assert len(bodies) == 32            # 2 types x 2 macro tiles x (plain 2 + signal 3 + scatter 3)
+    for name, ins in bodies.items():
+        assert sum(i.startswith("v_mfma") for i in ins) > 0
+        waited = None                   # wait states since the last MFMA of this straight-line stretch
+        for i in ins:
+            if i.endswith(":") or i.startswith(("s_branch", "s_cbranch", "s_endpgm")):
+                waited = None           # a new stretch: what ran before it is not known here
+                continue
+            if i.startswith("v_mfma"):
+                waited = 0
+                continue
+            if waited is not None:
+                if AGPR.search(i):
+                    assert waited >= MIN_WAIT_STATES, f"{name}: '{i}' only {waited} wait states behind an MFMA"
+                m = re.match(r"s_nop (\d+)", i)
+                waited += int(m.group(1)) + 1 if m else 1
+
+
+def test_register_budget_and_no_spills(gemm_asm):
+    _, meta = _kernels(gemm_asm)
+    assert len(meta) == 32
+    for name, m in meta.items():
+        assert m["spill"] == 0, f"{name} spills {m['spill']} registers"
+        # 512 registers per SIMD lane: what the GEMM leaves free is all the consumer's wavefronts
+        # (fewer than 64 registers each) have while they run beside it
+        assert m["vgpr"] <= 448, f"{name} takes {m['vgpr']} of 512 registers"

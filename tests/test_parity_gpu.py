@@ -338,6 +338,63 @@ def test_scatter_epilogue_and_reducescatter_slices(L, dev, comm_stream, ws, cseg
     assert torch.equal(one.cpu(), O.consume_reducescatter(want, cseg, BM, BN, ws)[1])
 
 
+# ---- matrix edges that are odd multiples of 128 -----------------------------------
+
+EDGE_SHAPES = [
+    (1152, 512, 72, 3),     # 128x256 layout tile, M = 9 x 128: the last macro row is half inside
+    (512, 640, 64, 5),      # 256x128 layout tile, N = 5 x 128: the last macro column is half inside
+    (2944, 2944, 64, 1),    # 128x128, 23 x 23 tiles on 256x256 macro tiles: both edges and the corner
+]
+
+
+@pytest.mark.parametrize("M,N,K,algo", EDGE_SHAPES)
+def test_half_macro_tiles_plain_signal_and_tickets(L, dev, M, N, K, algo):
+    """M and N only have to be multiples of the layout tile, as in the reference
+    (RA is [M/BM, N/BN], test/test.py:72-92); the 256x256 macro tile of this
+    kernel then hangs over the edge and must store and signal only what is inside."""
+    _say("edge", M, N, K, algo)
+    BM, BN, _ = capi.algo_tile(algo)
+    T = (M // BM) * (N // BN)
+    hint = tiling.raster_hint(M, N, algo)
+    assert sorted(hint) == list(range(T))                    # every layout tile issued exactly once
+    cseg = O.uniform_cseg(T, 7)
+    p = Path(L, dev, torch.bfloat16, M, N, K, algo, cseg=cseg, hint=hint, integer_inputs=True, seed=13)
+    p.build_table()
+    guard = 4096                                             # nothing may be written past the outputs
+    nat = torch.full((M * N + guard,), 7.0, dtype=p.dt, device=dev)
+    p.gemm_plain(out=nat)
+    p.dC = torch.full((M * N + guard,), 7.0, dtype=p.dt, device=dev)
+    p.gemm_signal()
+    torch.cuda.synchronize()
+    want = O.gemm(p.A, p.B)
+    assert torch.equal(nat[:M * N].cpu().view(M, N), want)
+    assert (nat[M * N:] == 7.0).all() and (p.dC[M * N:] == 7.0).all()
+    assert torch.equal(p.dC[:M * N].cpu(), O.place_tiles(want, p.ra_host.numpy(), BM, BN, 1))
+    assert p.dMM.cpu()[:p.G].tolist() == cseg and p.dMM.cpu()[p.G:].sum() == 0
+    # monitor mode: one ticket per layout tile, none for the parts outside
+    TN = N // BN
+    m = Path(L, dev, torch.bfloat16, M, N, K, algo, cseg=[T], hint=hint, monitor=True, integer_inputs=True, seed=13)
+    m.gemm_signal(use_table=False)
+    torch.cuda.synchronize()
+    mm = m.dMM.cpu()
+    assert sorted(mm[TN:].tolist()) == list(range(T)) and mm[TN - 1] == T and mm[0] == T
+
+
+def test_half_macro_tiles_scatter(L, dev):
+    M, N, K, algo, ws = 1152, 1024, 64, 3, 4     # 9 x 4 tiles of 128x256 -> 5 x 4 macro tiles, the last row half inside
+    BM, BN, _ = capi.algo_tile(algo)
+    T = (M // BM) * (N // BN)
+    _say("edge scatter", M, N, K)
+    cseg = O.uniform_cseg(T, 20)
+    p = Path(L, dev, torch.float16, M, N, K, algo, cseg=cseg, ws=ws, integer_inputs=True, seed=17)
+    p.build_table()
+    p.gemm_signal()
+    torch.cuda.synchronize()
+    want = O.scatter_place(O.gemm(p.A, p.B), p.ra_host.numpy(), p.re_host.numpy(), BM, BN, 1)
+    assert torch.equal(p.dC.cpu(), want)
+    assert p.dMM.cpu()[:p.G].tolist() == cseg
+
+
 # ---- wait / consume ------------------------------------------------------------
 
 def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
