@@ -78,6 +78,25 @@ def test_no_accumulator_access_close_behind_an_mfma(gemm_asm):
                 waited += int(m.group(1)) + 1 if m else 1
 
 
+def test_no_mfma_close_behind_an_accumulator_write(gemm_asm):
+    """The other direction: the zeroed accumulators must have landed before the first MFMA adds to them."""
+    bodies, _ = _kernels(gemm_asm)
+    for name, ins in bodies.items():
+        since_write = None
+        for i in ins:
+            if i.endswith(":") or i.startswith(("s_branch", "s_cbranch", "s_endpgm")):
+                since_write = None
+                continue
+            if i.startswith(("v_accvgpr_write", "v_accvgpr_mov")):
+                since_write = 0
+                continue
+            if since_write is not None:
+                if i.startswith("v_mfma"):
+                    assert since_write >= 4, f"{name}: an MFMA {since_write} wait states behind an accumulator write"
+                m = re.match(r"s_nop (\d+)", i)
+                since_write += int(m.group(1)) + 1 if m else 1
+
+
 def test_register_budget_and_no_spills(gemm_asm):
     _, meta = _kernels(gemm_asm)
     assert len(meta) == 32
