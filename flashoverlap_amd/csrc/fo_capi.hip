@@ -153,14 +153,41 @@ int fo_stream_sync(void* stream) {
     return FO_OK;
 }
 
+// Creating and destroying an event costs the host some 20 us a time, more than
+// the rest of a join: every thread keeps a few events per device and takes
+// them in turn.  A wait refers to the record that preceded it, so recording an
+// event again later does not disturb waits already enqueued on it.
+namespace {
+constexpr int kMaxDevices = 16, kEventsPerDevice = 4;
+struct JoinEvents {
+    hipEvent_t ev[kMaxDevices][kEventsPerDevice] = {};
+    unsigned next[kMaxDevices] = {};
+    // never destroyed: a thread may end after the runtime has shut down
+};
+thread_local JoinEvents t_join_events;
+}  // namespace
+
 int fo_stream_join(void* signaller, void* waiter) {
+    int dev = 0;
+    FO_HIP(hipGetDevice(&dev));
     hipEvent_t ev;
-    FO_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    const bool pooled = dev >= 0 && dev < kMaxDevices;
+    if (pooled) {
+        hipEvent_t& slot = t_join_events.ev[dev][t_join_events.next[dev]++ % kEventsPerDevice];
+        if (!slot) FO_HIP(hipEventCreateWithFlags(&slot, hipEventDisableTiming));
+        ev = slot;
+    } else {
+        FO_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    }
     hipError_t e = hipEventRecord(ev, (hipStream_t)signaller);
     if (e == hipSuccess) e = hipStreamWaitEvent((hipStream_t)waiter, ev, 0);
-    hipError_t d = hipEventDestroy(ev);
+    if (!pooled) {
+        hipError_t d = hipEventDestroy(ev);
+        FO_HIP(e);
+        FO_HIP(d);
+        return FO_OK;
+    }
     FO_HIP(e);
-    FO_HIP(d);
     return FO_OK;
 }
 
