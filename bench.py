@@ -114,6 +114,11 @@ def main() -> int:
     ap.add_argument("--no-overlap", action="store_true",
                     help="order the consumer behind the GEMM in the timed step (needed under counter collection, "
                          "which runs one kernel at a time)")
+    ap.add_argument("--fork", action="store_true",
+                    help="order the second stream behind the main stream before the GEMM, which OverlapImpl does when "
+                         "the call is being captured into a graph (costs 5-9 us of a step when done eagerly)")
+    ap.add_argument("--tune", action="append", default=[], metavar="KNOB=VALUE",
+                    help="library knob for this run (fo_tune: store_mode, release_mode, copy_streaming_stores)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build drives one GPU only; run with --gpus 1 "
@@ -127,6 +132,9 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     L = capi.lib()
+    for kv in a.tune:
+        knob, _, val = kv.partition("=")
+        capi.check(L.fo_tune(knob.encode(), int(val)))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     cu, khz, xcd = C.c_int(), C.c_int(), C.c_int()
@@ -244,9 +252,7 @@ def main() -> int:
                                             1, RA.data_ptr(), eps, main_stream))
 
     def step(g, overlap=True, ev=None):
-        if overlap and (g.G > 1 or not g.per_group):
-            # like OverlapImpl: the second stream's part of the step is ordered behind what the main stream
-            # held before the GEMM (a fork, so that the step is a fork/join pattern on the main stream)
+        if overlap and a.fork and (g.G > 1 or not g.per_group):
             capi.check(L.fo_stream_join(main_stream, comm))
         if ev:
             tm.record(ev[0])

@@ -191,6 +191,14 @@ int fo_stream_join(void* signaller, void* waiter) {
     return FO_OK;
 }
 
+int fo_stream_is_capturing(void* stream, int* capturing) {
+    if (!capturing) return fail(FO_ERR_ARG, "fo_stream_is_capturing: null output");
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    FO_HIP(hipStreamIsCapturing((hipStream_t)stream, &status));
+    *capturing = status == hipStreamCaptureStatusActive;
+    return FO_OK;
+}
+
 int fo_event_create(void** ev) {
     if (!ev) return fail(FO_ERR_ARG, "fo_event_create: null output");
     hipEvent_t e;

@@ -676,7 +676,7 @@ int tune(const char* key, int value) {
     const std::string_view k(key);
     if (k == "store_mode") g_store_mode = value ? 1 : 0;
     else if (k == "release_mode") g_release_mode = value ? 1 : 0;
-    else if (k == "copy_streaming_stores") g_copy_streaming_stores = value ? 1 : 0;
+    else if (k == "copy_streaming_stores" && value >= 0 && value <= 2) g_copy_streaming_stores = value;
     else return fail(FO_ERR_ARG, "fo_tune: unknown knob '%s'", key);
     return FO_OK;
 }

@@ -24,7 +24,7 @@ namespace fo {
 __device__ int g_wait_timeouts = 0;
 
 static int g_timeout_ms = 10000;
-int g_copy_streaming_stores = 0;   // fo_tune "copy_streaming_stores": non-temporal stores in the consumer copy
+int g_copy_streaming_stores = 2;   // fo_tune "copy_streaming_stores": 0 never, 1 always, 2 chosen per launch
 
 // Bounded poll of *addr until pred(value); returns false on expiry.
 template <typename Pred>
@@ -64,14 +64,16 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // kCopyUnroll loads in flight.  COHERENT: read with agent-scope loads that do
 // not hit in the non-coherent caches (for data another XCD wrote while this
 // kernel runs).  The loads are non-temporal: the source streams through once.
-// The stores are ordinary ones by default, so that the destination can stay in
-// the 256 MB memory-side cache for the kernel that reads it next (on some
-// machines reorder+RMSNorm took 30 us instead of 24 right behind a copy with
-// non-temporal stores); streaming_stores != 0 makes them non-temporal, which
-// keeps the copy from displacing other data in that cache.
-template <bool COHERENT, int WIDTH>
+// STREAM: the stores are non-temporal too, which keeps the copy from displacing
+// the operands of a GEMM running beside it from the 256 MB memory-side cache
+// (with ordinary stores an overlapped 16384x8192x1024 GEMM ran 4 % longer);
+// without it the destination may stay in that cache for the kernel that reads
+// it next (reorder+RMSNorm right behind a copy took 25 us instead of 31).  A
+// compile-time choice: as a run-time branch around the two kinds of store the
+// compiler merges them into one ordinary store.
+template <bool COHERENT, int WIDTH, bool STREAM>
 __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __restrict__ d, long long n, int me,
-                                          int team, int t, int streaming_stores) {
+                                          int team, int t) {
     const long long chunk = (long long)WIDTH * kCopyUnroll;
     [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc;
     if constexpr (COHERENT) rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, 0xffffffff, 0x00020000);
@@ -89,7 +91,7 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
         for (int u = 0; u < kCopyUnroll; ++u) {
             const long long i = base + u * WIDTH + t;
             if (i < n) {
-                if (streaming_stores) __builtin_nontemporal_store(v[u], (u32x4*)(d + i));
+                if constexpr (STREAM) __builtin_nontemporal_store(v[u], (u32x4*)(d + i));
                 else *(u32x4*)(d + i) = v[u];
             }
         }
@@ -117,10 +119,11 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
 // registers, and these wavefronts have to fit beside it.  Each wavefront finds
 // its groups on its own: 64 groups at a time, one per lane, with wavefront
 // scans for the group offsets and the team windows.
+template <bool STREAM>
 __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
     const int* __restrict__ cseg, int G, int* MM, const uint4* __restrict__ src, uint4* __restrict__ dst,
     long long tile_units, int nslices, int slice_first, int slice_count, long long slice_stride_units,
-    int* order_log, long long ticks, int streaming_stores) {
+    int* order_log, long long ticks) {
     const int lane = threadIdx.x & 63;
     const int self = __builtin_amdgcn_readfirstlane((int)blockIdx.x * kWavesPerBlock + (int)(threadIdx.x >> 6));
     const int members = (int)gridDim.x * kWavesPerBlock;
@@ -180,18 +183,18 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
             if (!__shfl(ok, 0, 64)) return;  // the wait expired: this wavefront gives up on the rest
             const long long part = tile_units * need / nslices;
             for (int k = 0; k < slice_count; ++k)
-                team_copy<true, 64>(src + glo + (slice_first + k) * part, dst + k * slice_stride_units + glo / nslices,
-                                    part, mem, tm, lane, streaming_stores);
+                team_copy<true, 64, STREAM>(src + glo + (slice_first + k) * part,
+                                            dst + k * slice_stride_units + glo / nslices, part, mem, tm, lane);
         }
         lo_base += __shfl(su, 63, 64);
         start_base = (int)(((long long)start_base + __shfl(st, 63, 64)) % members);
     }
 }
 
+template <bool STREAM>
 __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                                long long units, const unsigned short* src_tail,
-                                                               unsigned short* dst_tail, int tail, int streaming_stores,
-                                                               int that, int* addr) {
+                                                               unsigned short* dst_tail, int tail, int that, int* addr) {
     // Settling a counter whose producer ran earlier on this stream takes no
     // waiting: it holds its final value.  The right value is cleared like
     // wait_kernel does; a wrong one is left and counted like an expired wait.
@@ -201,7 +204,7 @@ __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __re
         else
             atomicAdd(&g_wait_timeouts, 1);
     }
-    team_copy<false, kCopyThreads>(src, dst, units, blockIdx.x, gridDim.x, threadIdx.x, streaming_stores);
+    team_copy<false, kCopyThreads, STREAM>(src, dst, units, blockIdx.x, gridDim.x, threadIdx.x);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
@@ -312,9 +315,9 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
         return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d outside 1..%d (one workgroup per CU)", nblocks, facts->cus);
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
-    hipLaunchKernelGGL(wait_consume_kernel, dim3(nblocks), dim3(64 * kWavesPerBlock), 0, stream, cseg, G, MM, (const uint4*)src,
-                       (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks,
-                       g_copy_streaming_stores);
+    auto kern = g_copy_streaming_stores ? wait_consume_kernel<true> : wait_consume_kernel<false>;   // runs beside the GEMM
+    hipLaunchKernelGGL(kern, dim3(nblocks), dim3(64 * kWavesPerBlock), 0, stream, cseg, G, MM, (const uint4*)src,
+                       (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }
@@ -330,9 +333,18 @@ int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream,
     size_t blocks = (units + per_block - 1) / per_block;
     if (blocks > 1024) blocks = 1024;
     if (blocks == 0) blocks = 1;
-    hipLaunchKernelGGL(consume_kernel, dim3((unsigned)blocks), dim3(kCopyThreads), 0, stream, (const uint4*)src,
+    // Automatic choice: a copy that settles its own counter follows its GEMM on the stream and is read
+    // next, so it stores normally.  Any other copy may run beside a GEMM; it is the large ones that
+    // push that GEMM's operands out of the memory-side cache (67 MB groups of a 16384x8192 output: the
+    // GEMM beside them ran 8 % longer with ordinary stores), while after a small one the reader finds
+    // the data still cached (33 MB groups of 8192x4096: reorder+RMSNorm 23 us against 31).
+    constexpr size_t kStreamFrom = 48u << 20;
+    const bool stream_stores =
+        g_copy_streaming_stores == 1 || (g_copy_streaming_stores == 2 && !addr && bytes >= kStreamFrom);
+    auto kern = stream_stores ? consume_kernel<true> : consume_kernel<false>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kCopyThreads), 0, stream, (const uint4*)src,
                        (uint4*)dst, (long long)units, (const unsigned short*)((const char*)src + units * 16),
-                       (unsigned short*)((char*)dst + units * 16), tail, g_copy_streaming_stores, that, addr);
+                       (unsigned short*)((char*)dst + units * 16), tail, that, addr);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }

@@ -136,10 +136,14 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host);
  *                  "store_mode" says.
  *   "store_mode"   with release_mode 0 only.  1 (default): write-through tile
  *                  stores; 0: cached tile stores.
- *   "copy_streaming_stores"  0 (default): the consumer copies (fo_consume,
- *                  fo_wait_consume) store with ordinary stores, so their
- *                  destination may stay in the memory-side cache for its
- *                  reader; 1: non-temporal stores. */
+ *   "copy_streaming_stores"  how the consumer copies store.  2 (default):
+ *                  chosen per launch: non-temporal stores in fo_wait_consume
+ *                  and in fo_consume calls of 48 MiB or more (copies of that
+ *                  size running beside a GEMM push its operands out of the
+ *                  memory-side cache), ordinary stores in smaller ones and in
+ *                  fo_settle_consume (their destination is then still cached
+ *                  for the kernel that reads it next); 1: non-temporal
+ *                  everywhere; 0: ordinary everywhere. */
 int fo_tune(const char* key, int value);
 
 /* ---- counting / wait -------------------------------------------------- */
@@ -236,6 +240,9 @@ int fo_stream_sync(void* stream);
 /* Make `waiter` wait for everything enqueued so far on `signaller`.  Replaces
  * the per-call event create/record/wait/destroy (src/overlap_impl.cu:267-270). */
 int fo_stream_join(void* signaller, void* waiter);
+/* *capturing = 1 while `stream` is recording into a graph (stream capture), else 0.
+ * No counterpart in the reference, whose overlapped call cannot be captured. */
+int fo_stream_is_capturing(void* stream, int* capturing);
 
 /* Timing helpers for harnesses that cannot use torch events on foreign
  * streams: opaque hipEvent_t handles. */

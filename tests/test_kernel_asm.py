@@ -105,3 +105,30 @@ def test_register_budget_and_no_spills(gemm_asm):
         # 512 registers per SIMD lane: what the GEMM leaves free is all the consumer's wavefronts
         # (fewer than 64 registers each) have while they run beside it
         assert m["vgpr"] <= 448, f"{name} takes {m['vgpr']} of 512 registers"
+
+
+def test_consumer_copy_variants_differ_in_their_stores(tmp_path):
+    """The two store policies of the consumer copy are separate kernels: written as one kernel
+    with a run-time branch the compiler folded both into ordinary stores and the knob did nothing."""
+    hipcc = os.path.join(build.ROCM, "bin", "hipcc")
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    out = tmp_path / "fo_sync.s"
+    flags = [f for f in build.HIPCC_FLAGS if f != "-fPIC"]
+    subprocess.run([hipcc, *flags, "--cuda-device-only", "-S", os.path.join(build.CSRC, "fo_sync.hip"), "-o", str(out)],
+                   check=True, capture_output=True, timeout=600)
+    stores = {}
+    name = None
+    for line in out.read_text().splitlines():
+        m = re.match(r"^(_ZN2fo\d+(?:consume_kernel|wait_consume_kernel)ILb([01])E\S*):", line)
+        if m:
+            name = m.group(1)
+            stores[name] = [m.group(2) == "1", 0, 0]
+            continue
+        if name and line.startswith(".Lfunc_end"):
+            name = None
+        if name and "global_store_dwordx4" in line:
+            stores[name][1 if re.search(r"\bnt\b", line.split(";")[0]) else 2] += 1
+    assert len(stores) == 4
+    for name, (stream, nt, plain) in stores.items():
+        assert (nt > 0 and plain == 0) if stream else (plain > 0 and nt == 0), (name, nt, plain)
