@@ -100,7 +100,7 @@ struct Mma<__bf16> {
 // from before that MFMA).
 static __device__ __forceinline__ float acc_read(const float& a) {
     float v;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));   // not volatile: free to be scheduled within the epilogue
     return v;
 }
 // More wait states than the longest MFMA needs before its result can be read.
@@ -488,6 +488,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     // acc[i][j][r] is element m = 16i + l%16, n = 16j + 4(l/16) + r (fr_g = l/16).
     __builtin_amdgcn_s_setprio(0);
     settle_mfma();
+    __builtin_amdgcn_sched_barrier(0);   // no accumulator read is scheduled ahead of the delay
     __syncthreads();  // every wave is done with the panel buffers
     constexpr int PITCH = WT * 2 + 16;                  // strip row pitch in bytes
     constexpr int ROWCH = WT / 8;                       // 16-byte chunks per strip row
