@@ -9,7 +9,7 @@ the staging buffer.
 
 Prints ONE JSON line.  `value` is 2*M*N*K divided by the whole step time.  The
 roofline object is for the dominant kernel (the signalling GEMM) as it ran
-inside the timed steps, from HIP events around every launch on its own stream.
+inside the timed steps, from a HIP event pair attached to every launch's own dispatch.
 The same run also times, back to back and on their own, the signalling GEMM
 and its plain twin (signal overhead), reorder+RMSNorm (HBM roofline; over a
 rotation of buffer pairs larger than the 256 MB memory-side cache, and inside
@@ -254,24 +254,20 @@ def main() -> int:
     def step(g, overlap=True, ev=None):
         if overlap and a.fork and (g.G > 1 or not g.per_group):
             capi.check(L.fo_stream_join(main_stream, comm))
-        if ev:
-            tm.record(ev[0])
+        if ev:   # the GEMM's own dispatch carries the two events: its duration without launch gaps
+            capi.check(L.fo_time_next_launch(ev[0], ev[1]))
         gemm_signal(g)
-        if ev:
-            tm.record(ev[1])
         if not overlap:  # consumer ordered behind the GEMM: the serial reference for the overlap
             capi.check(L.fo_stream_join(main_stream, comm))
         wait_consume(g)
         if ev and len(ev) > 2:
-            tm.record(ev[2])   # fires once the last group has been consumed
+            capi.check(L.fo_time_next_launch(ev[2], ev[3]))
         norm()
-        if ev and len(ev) > 2:
-            tm.record(ev[3])
 
     def time_steps(g, overlap, probes=2):
         """Wall time per step and the duration of the signalling GEMM inside those same steps (one HIP
-        event pair per step on the stream it runs on); with probes=4 also the duration of
-        reorder+RMSNorm (a second pair per step; every pair costs the step a few microseconds)."""
+        event pair per step, attached to the kernel's own dispatch: what a kernel trace reports, no launch
+        gaps and no extra packets in the stream); with probes=4 also the duration of reorder+RMSNorm."""
         evs = [tuple(tm.event() for _ in range(probes)) for _ in range(a.steps)]
         for _ in range(a.warmup):
             step(g, overlap)

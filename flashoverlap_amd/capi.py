@@ -44,6 +44,7 @@ SIGNATURES = {
     "fo_stream_sync": (_i, [_vp]),
     "fo_stream_join": (_i, [_vp, _vp]),
     "fo_stream_is_capturing": (_i, [_vp, C.POINTER(C.c_int)]),
+    "fo_time_next_launch": (_i, [_vp, _vp]),
     "fo_event_create": (_i, [C.POINTER(_vp)]),
     "fo_event_destroy": (_i, [_vp]),
     "fo_event_record": (_i, [_vp, _vp]),

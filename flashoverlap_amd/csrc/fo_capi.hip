@@ -28,6 +28,8 @@ static const int kAlgo[][3] = {
 };
 constexpr int kAlgoCount = sizeof(kAlgo) / sizeof(kAlgo[0]);
 
+thread_local LaunchTimer t_launch_timer;
+
 int algo_tile(int algo, int* BM, int* BN, int* BK) {
     if (algo < 0 || algo >= kAlgoCount) return FO_ERR_ARG;
     *BM = kAlgo[algo][0];
@@ -188,6 +190,13 @@ int fo_stream_join(void* signaller, void* waiter) {
         return FO_OK;
     }
     FO_HIP(e);
+    return FO_OK;
+}
+
+int fo_time_next_launch(void* start_event, void* stop_event) {
+    if (!start_event != !stop_event) return fail(FO_ERR_ARG, "fo_time_next_launch: pass both events or neither");
+    t_launch_timer.start = (hipEvent_t)start_event;
+    t_launch_timer.stop = (hipEvent_t)stop_event;
     return FO_OK;
 }
 

@@ -53,6 +53,7 @@
 // and src/overlap/gemm_with_scatter.h:146-196; the kernel itself shares nothing
 // with the reference's MUTlass mainloop.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <atomic>
 #include <string_view>
@@ -579,7 +580,13 @@ static int launch_one(const GemmParams& p, hipStream_t stream) {
         FO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes));
         configured.fetch_or(bit, std::memory_order_release);
     }
-    hipLaunchKernelGGL(kern, dim3(p.GM * p.GN), dim3(256), smem_bytes, stream, p);
+    if (t_launch_timer.start) {
+        const LaunchTimer t = t_launch_timer;
+        t_launch_timer = LaunchTimer{};
+        hipExtLaunchKernelGGL(kern, dim3(p.GM * p.GN), dim3(256), smem_bytes, stream, t.start, t.stop, 0, p);
+    } else {
+        hipLaunchKernelGGL(kern, dim3(p.GM * p.GN), dim3(256), smem_bytes, stream, p);
+    }
     FO_HIP(hipGetLastError());
     return FO_OK;
 }

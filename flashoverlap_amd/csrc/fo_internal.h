@@ -21,6 +21,14 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
 int algo_tile(int algo, int* BM, int* BN, int* BK);
 
+// fo_time_next_launch: a pair of events that the next GEMM or RMSNorm launch of this thread
+// attaches to its own dispatch, so that the time between them is the kernel's, without the
+// launch gaps an event pair recorded around the launch includes.  Taken by the launch that uses it.
+struct LaunchTimer {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+extern thread_local LaunchTimer t_launch_timer;
+
 // fo_gemm.hip
 int choose_macro_tile(int BM, int BN, int M, int N);
 int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg, int G,

@@ -15,6 +15,7 @@
 // of two 16-bit floats is exact in fp32, so rounding it once equals the
 // reference's half-precision multiply).  eps is a parameter here.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include "fo_internal.h"
 
@@ -155,9 +156,17 @@ static int launch_t(const void* x, const void* gamma, void* out, const int* RA, 
                     hipStream_t stream) {
     const int ch = (p.dim / 8 + 63) / 64;
     const dim3 grid((p.bs + kRowsPerBlock - 1) / kRowsPerBlock, nbatch), block(64 * kRowsPerBlock);
-#define FO_RMS_CASE(CH)                                                                                       \
-    hipLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, 0, stream, (const T*)x, (const T*)gamma, \
-                       (T*)out, RA, p)
+    const LaunchTimer timer = t_launch_timer;
+    t_launch_timer = LaunchTimer{};
+#define FO_RMS_CASE(CH)                                                                                           \
+    do {                                                                                                          \
+        if (timer.start)                                                                                          \
+            hipExtLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, 0, stream, timer.start, timer.stop, \
+                                  0, (const T*)x, (const T*)gamma, (T*)out, RA, p);                               \
+        else                                                                                                      \
+            hipLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, 0, stream, (const T*)x,                \
+                               (const T*)gamma, (T*)out, RA, p);                                                  \
+    } while (0)
     if (ch <= 1) FO_RMS_CASE(1);
     else if (ch <= 2) FO_RMS_CASE(2);
     else if (ch <= 4) FO_RMS_CASE(4);

@@ -240,6 +240,12 @@ int fo_stream_sync(void* stream);
 /* Make `waiter` wait for everything enqueued so far on `signaller`.  Replaces
  * the per-call event create/record/wait/destroy (src/overlap_impl.cu:267-270). */
 int fo_stream_join(void* signaller, void* waiter);
+/* Measurement aid, no counterpart in the reference: the next fo_gemm*, fo_rmsnorm* or
+ * fo_reorder_rmsnorm* launch made by the calling thread attaches the two events (from
+ * fo_event_create) to its own dispatch; fo_event_elapsed_ms between them is then the
+ * kernel's duration, as a profiler reports it, without the launch gaps that an event
+ * pair recorded around the call includes.  Passing two nulls cancels. */
+int fo_time_next_launch(void* start_event, void* stop_event);
 /* *capturing = 1 while `stream` is recording into a graph (stream capture), else 0.
  * No counterpart in the reference, whose overlapped call cannot be captured. */
 int fo_stream_is_capturing(void* stream, int* capturing);
