@@ -164,6 +164,35 @@ def test_gemm_random_within_tolerance(L, dev, dt, K):
     assert ((got.float() - gated.float()).abs() <= ulp * gated.float().abs() + 1e-6).all()
 
 
+def test_time_next_launch_gives_the_kernel_duration(L, dev):
+    """Events attached to the dispatch bracket the kernel alone: a positive time, no longer than
+    what an event pair recorded around the call measures; the pair is used up by one launch."""
+    p = Path(L, dev, torch.bfloat16, 2048, 2048, 2048, 1, seed=1)
+    out = torch.zeros(2048, 2048, dtype=p.dt, device=dev)
+    p.gemm_plain(out=out)
+    torch.cuda.synchronize()
+    evs = [C.c_void_p() for _ in range(4)]
+    for e in evs:
+        capi.check(L.fo_event_create(C.byref(e)))
+    inner0, inner1, outer0, outer1 = evs
+    capi.check(L.fo_event_record(outer0, None))
+    capi.check(L.fo_time_next_launch(inner0, inner1))
+    p.gemm_plain(out=out)
+    capi.check(L.fo_event_record(outer1, None))
+    p.gemm_plain(out=out)                      # not timed: the pair was taken by the launch before
+    torch.cuda.synchronize()
+    t_in, t_out = C.c_float(), C.c_float()
+    capi.check(L.fo_event_elapsed_ms(inner0, inner1, C.byref(t_in)))
+    capi.check(L.fo_event_elapsed_ms(outer0, outer1, C.byref(t_out)))
+    _say("  kernel %.1f us inside a bracket of %.1f us" % (t_in.value * 1e3, t_out.value * 1e3))
+    flops = 2.0 * 2048 ** 3
+    assert 0 < t_in.value <= t_out.value
+    assert flops / (t_in.value * 1e-3) < 2.6e15          # not faster than the chip
+    assert L.fo_time_next_launch(inner0, None) == capi.FO_ERR_ARG
+    for e in evs:
+        capi.check(L.fo_event_destroy(e))
+
+
 def test_gemm_rejects_unsupported_shapes(L, dev):
     a = torch.zeros(384, 384, dtype=torch.float16, device=dev)  # large enough for every call below
     assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 44, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
