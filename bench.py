@@ -217,6 +217,10 @@ def main() -> int:
                                          None, a.consumer_blocks, comm))
             capi.check(L.fo_stream_join(comm, main_stream))
             return
+        # like OverlapImpl: the groups before the last are copied beside the GEMM; if that is a lot of data,
+        # with non-temporal stores (1), else with ordinary ones (2); the last group always with ordinary ones
+        beside = 2 * BM * BN * sum(g.cseg[:-1])
+        beside_policy = 1 if beside >= (64 << 20) else 2
         acc = 0
         for gi, n in enumerate(g.cseg):
             stream = comm
@@ -231,13 +235,10 @@ def main() -> int:
                 capi.check(L.fo_wait(n, g.MM.data_ptr() + 4 * gi, stream))
             elems = n * BM * BN
             part = elems // ws
-            for k in range(ws):  # ws > 1: slice k of the group goes to rank k's receive buffer
-                src = Cp.data_ptr() + 2 * (acc + k * part)
-                dst = staging.data_ptr() + 2 * (k * (M * N // ws) + acc // ws)
-                if settle and k == 0:
-                    capi.check(L.fo_settle_consume(n, g.MM.data_ptr() + 4 * gi, src, dst, 2 * part, stream))
-                else:
-                    capi.check(L.fo_consume(src, dst, 2 * part, stream))
+            # one launch per group (ws > 1: slice k of the group goes to rank k's receive buffer)
+            capi.check(L.fo_consume_slices(n, g.MM.data_ptr() + 4 * gi if settle else None, Cp.data_ptr() + 2 * acc,
+                                           staging.data_ptr() + 2 * (acc // ws), 2 * part, ws, 2 * (M * N // ws),
+                                           2 if gi == g.G - 1 else beside_policy, stream))
             acc += elems
         if a.last_group == "comm" or (a.last_group == "settle_then_join" and g.G > 1):
             capi.check(L.fo_stream_join(comm, main_stream))

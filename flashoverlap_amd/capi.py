@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfo_hip.so")
 
 FO_F16, FO_BF16 = 0, 1
 FO_OK, FO_ERR_ARG, FO_ERR_SHAPE, FO_ERR_HIP, FO_ERR_TIMEOUT, FO_ERR_LIMIT = range(6)
+FO_COPY_AUTO, FO_COPY_STREAM, FO_COPY_CACHED = range(3)   # store policy of fo_consume_slices
 
 _vp, _ip, _i, _ll, _sz, _f = C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_longlong, C.c_size_t, C.c_float
 
@@ -36,6 +37,7 @@ SIGNATURES = {
     "fo_wait_timeouts": (_i, [_ip, _i]),
     "fo_consume": (_i, [_vp, _vp, _sz, _vp]),
     "fo_settle_consume": (_i, [_i, _vp, _vp, _vp, _sz, _vp]),
+    "fo_consume_slices": (_i, [_i, _vp, _vp, _vp, _sz, _i, _sz, _i, _vp]),
     "fo_reorder_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "fo_reorder_rmsnorm_batched": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "fo_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _f, _vp]),

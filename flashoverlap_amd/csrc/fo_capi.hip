@@ -121,6 +121,12 @@ int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t by
     return launch_consume(src, dst, bytes, (hipStream_t)stream, that, addr);
 }
 
+int fo_consume_slices(int that, int* addr, const void* src, void* dst, size_t slice_bytes, int nslices,
+                      size_t dst_stride_bytes, int store_policy, void* stream) {
+    return launch_consume(src, dst, slice_bytes, (hipStream_t)stream, that, addr, nslices, dst_stride_bytes,
+                          store_policy);
+}
+
 int fo_reorder_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,
                        int rldn, const int* RA, float eps, void* stream) {
     if (!RA) return fail(FO_ERR_ARG, "fo_reorder_rmsnorm: null RA");

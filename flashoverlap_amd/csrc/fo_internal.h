@@ -47,7 +47,8 @@ int launch_wait(int that, int* addr, hipStream_t stream);
 int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* dst, long long tile_elems,
                         int nslices, int slice_first, int slice_count, long long slice_stride, int* order_log,
                         int nblocks, hipStream_t stream);
-int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream, int that = 0, int* addr = nullptr);
+int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream, int that = 0, int* addr = nullptr,
+                   int nslices = 1, size_t dst_stride_bytes = 0, int policy = FO_COPY_AUTO);
 int set_wait_timeout_ms(int ms);
 int wait_timeouts(int* count, int reset);
 

@@ -191,21 +191,25 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
     }
 }
 
+// blockIdx.y is the slice: slice k of the source lies k * units behind the first, slice k of
+// the destination k * dst_stride_units (the receive buffers of a ReduceScatter, side by side).
 template <bool STREAM>
 __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
-                                                               long long units, const unsigned short* src_tail,
-                                                               unsigned short* dst_tail, int tail, int that, int* addr) {
+                                                               long long units, long long dst_stride_units,
+                                                               const unsigned short* src_tail, unsigned short* dst_tail,
+                                                               int tail, int that, int* addr) {
     // Settling a counter whose producer ran earlier on this stream takes no
     // waiting: it holds its final value.  The right value is cleared like
     // wait_kernel does; a wrong one is left and counted like an expired wait.
-    if (addr && blockIdx.x == 0 && threadIdx.x == 0) {
+    if (addr && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
         if (__hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == that)
             __hip_atomic_store(addr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else
             atomicAdd(&g_wait_timeouts, 1);
     }
-    team_copy<false, kCopyThreads, STREAM>(src, dst, units, blockIdx.x, gridDim.x, threadIdx.x);
-    if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
+    team_copy<false, kCopyThreads, STREAM>(src + blockIdx.y * units, dst + blockIdx.y * dst_stride_units, units,
+                                           blockIdx.x, gridDim.x, threadIdx.x);
+    if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];   // one slice only
 }
 
 // table[s] = number of inclusive prefix sums of cseg that are <= s, i.e. what
@@ -322,28 +326,38 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
     return FO_OK;
 }
 
-int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream, int that, int* addr) {
+int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream, int that, int* addr, int nslices,
+                   size_t dst_stride_bytes, int policy) {
+    const char* who = nslices > 1 ? "fo_consume_slices" : "fo_consume";
+    if (nslices <= 0 || nslices > 65535) return fail(FO_ERR_ARG, "%s: %d slices outside 1..65535", who, nslices);
     if (bytes == 0 && !addr) return FO_OK;
-    if (!src || !dst) return fail(FO_ERR_ARG, "fo_consume: null buffer");
-    if (bytes & 1) return fail(FO_ERR_ARG, "fo_consume: %zu bytes is not a whole number of 16-bit elements", bytes);
-    if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "fo_consume: buffers must be 16-byte aligned");
+    if (!src || !dst) return fail(FO_ERR_ARG, "%s: null buffer", who);
+    if (bytes & 1) return fail(FO_ERR_ARG, "%s: %zu bytes is not a whole number of 16-bit elements", who, bytes);
+    if (((uintptr_t)src | (uintptr_t)dst) & 15) return fail(FO_ERR_ARG, "%s: buffers must be 16-byte aligned", who);
+    if (nslices > 1 && ((bytes | dst_stride_bytes) & 15))
+        return fail(FO_ERR_SHAPE, "%s: slices of %zu bytes, %zu apart, are not whole 16-byte units", who, bytes, dst_stride_bytes);
     const size_t units = bytes / 16;
     const int tail = (int)((bytes % 16) / 2);
     const size_t per_block = (size_t)kCopyThreads * kCopyUnroll;
     size_t blocks = (units + per_block - 1) / per_block;
-    if (blocks > 1024) blocks = 1024;
+    const size_t most = 1024 / (size_t)(nslices < 1024 ? nslices : 1024);   // about 1024 workgroups over all slices
+    if (blocks > most) blocks = most;
     if (blocks == 0) blocks = 1;
-    // Automatic choice: a copy that settles its own counter follows its GEMM on the stream and is read
-    // next, so it stores normally.  Any other copy may run beside a GEMM; it is the large ones that
-    // push that GEMM's operands out of the memory-side cache (67 MB groups of a 16384x8192 output: the
-    // GEMM beside them ran 8 % longer with ordinary stores), while after a small one the reader finds
-    // the data still cached (33 MB groups of 8192x4096: reorder+RMSNorm 23 us against 31).
+    // Store policy.  What matters is how much is copied while a GEMM runs beside the copies: from some
+    // tens of MB on, ordinary stores push that GEMM's operands out of the memory-side cache (c4, 201 MB
+    // beside the GEMM: it ran 8 % longer; c5, 100 MB: 4 %), below that the reader of the destination
+    // gains more from finding it still cached (c3, 33 MB: reorder+RMSNorm 23 us against 31).  A caller
+    // that knows the whole call says which it wants; left to itself a launch goes by its own size, and
+    // one that settles its own counter follows its GEMM and is read next, so it stores normally.
+    if (policy < FO_COPY_AUTO || policy > FO_COPY_CACHED) return fail(FO_ERR_ARG, "%s: store policy %d", who, policy);
     constexpr size_t kStreamFrom = 48u << 20;
-    const bool stream_stores =
-        g_copy_streaming_stores == 1 || (g_copy_streaming_stores == 2 && !addr && bytes >= kStreamFrom);
+    bool stream_stores = policy == FO_COPY_STREAM ||
+                         (policy == FO_COPY_AUTO && !addr && bytes * (size_t)nslices >= kStreamFrom);
+    if (g_copy_streaming_stores != 2) stream_stores = g_copy_streaming_stores == 1;   // forced by fo_tune
     auto kern = stream_stores ? consume_kernel<true> : consume_kernel<false>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kCopyThreads), 0, stream, (const uint4*)src,
-                       (uint4*)dst, (long long)units, (const unsigned short*)((const char*)src + units * 16),
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks, (unsigned)nslices), dim3(kCopyThreads), 0, stream, (const uint4*)src,
+                       (uint4*)dst, (long long)units, (long long)(dst_stride_bytes / 16),
+                       (const unsigned short*)((const char*)src + units * 16),
                        (unsigned short*)((char*)dst + units * 16), tail, that, addr);
     FO_HIP(hipGetLastError());
     return FO_OK;

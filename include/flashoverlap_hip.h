@@ -204,6 +204,25 @@ int fo_consume(const void* src, void* dst, size_t bytes, void* stream);
  * src/overlap_impl.cu:257-265, and then joins the streams). */
 int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t bytes, void* stream);
 
+/* One launch for the `nslices` slices of a released group: slice k is the
+ * `slice_bytes` bytes at src + k * slice_bytes and goes to dst + k *
+ * dst_stride_bytes.  The one-GPU stand-in for one mcclReduceScatter call on a
+ * group when all ranks' receive buffers are kept side by side
+ * (src/overlap_impl.cu:319-320 makes one collective call per group, not one per
+ * rank).  addr != NULL: also settle the group's counter like fo_settle_consume
+ * (for the last group, on the GEMM's stream); addr == NULL: a plain copy.
+ * store_policy: FO_COPY_STREAM = non-temporal stores (for copies that run
+ * beside a GEMM when the call copies tens of MB that way: they then leave its
+ * operands in the memory-side cache), FO_COPY_CACHED = ordinary stores (the
+ * destination stays cached for its reader), FO_COPY_AUTO = by the size of this
+ * launch alone, as fo_consume does.  fo_tune("copy_streaming_stores", 0 or 1)
+ * overrides all three. */
+#define FO_COPY_AUTO 0
+#define FO_COPY_STREAM 1
+#define FO_COPY_CACHED 2
+int fo_consume_slices(int that, int* addr, const void* src, void* dst, size_t slice_bytes, int nslices,
+                      size_t dst_stride_bytes, int store_policy, void* stream);
+
 /* ---- RMSNorm ---------------------------------------------------------- */
 
 /* out[b,:] = rmsnorm(gather(x)[b,:]) * gamma, gather as in the layout header.

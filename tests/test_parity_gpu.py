@@ -472,6 +472,35 @@ def test_settle_consume_clears_the_right_count_and_reports_a_wrong_one(L, dev, c
     assert L.fo_settle_consume(0, None, src.data_ptr(), dst.data_ptr(), 16, comm_stream) == capi.FO_ERR_ARG
 
 
+def test_consume_slices_equals_one_copy_per_slice(L, dev, comm_stream):
+    """One launch for all ranks' slices of a group (one collective call per group,
+    src/overlap_impl.cu:319-320) against fo_consume slice by slice."""
+    ws, part, stride = 8, 4096 * 5, 40000            # elements; stride > part: gaps between the receive buffers
+    src = torch.randint(-30000, 30000, (ws * part + 64,), dtype=torch.int16, device=dev)
+    want = torch.full((ws * stride,), -1, dtype=torch.int16, device=dev)
+    got = want.clone()
+    for k in range(ws):
+        capi.check(L.fo_consume(src.data_ptr() + 2 * (64 + k * part), want.data_ptr() + 2 * k * stride, 2 * part,
+                                comm_stream))
+    capi.check(L.fo_consume_slices(0, None, src.data_ptr() + 2 * 64, got.data_ptr(), 2 * part, ws, 2 * stride,
+                                   capi.FO_COPY_STREAM, comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert torch.equal(got, want)
+    assert (got.view(ws, stride)[:, part:] == -1).all()      # nothing written between the slices
+    # with a counter: settled once, by the launch as a whole
+    mm = torch.tensor([5], dtype=torch.int32, device=dev)
+    got.fill_(-1)
+    capi.check(L.fo_consume_slices(5, mm.data_ptr(), src.data_ptr() + 2 * 64, got.data_ptr(), 2 * part, ws, 2 * stride,
+                                   capi.FO_COPY_CACHED, comm_stream))
+    capi.check(L.fo_stream_sync(comm_stream))
+    assert torch.equal(got, want) and mm.item() == 0 and _timeouts(L) == 0
+    # slices that are not whole 16-byte units are refused
+    assert L.fo_consume_slices(0, None, src.data_ptr(), got.data_ptr(), 2 * 4100, 2, 2 * stride, capi.FO_COPY_AUTO,
+                               comm_stream) == capi.FO_ERR_SHAPE
+    assert L.fo_consume_slices(0, None, src.data_ptr(), got.data_ptr(), 2 * 4096, 2, 2 * stride, 7,
+                               comm_stream) == capi.FO_ERR_ARG
+
+
 def test_consume_copies_exactly_the_bytes(L, dev):
     src = torch.randint(-30000, 30000, (100003,), dtype=torch.int16, device=dev)
     for off, n in ((0, 100003), (8, 77), (16, 8), (24, 4099)):
