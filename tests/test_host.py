@@ -95,6 +95,21 @@ def test_raster_xcd_locality():
         assert len(rows) * len(cols) == 32 and len(rows) <= 8
 
 
+@pytest.mark.parametrize("M,N", [(8192, 4096), (16384, 8192), (8192, 8192), (4096, 4096)])
+def test_raster_waves_finish_whole_rows(M, N):
+    """A hardware wave is 256 workgroups; with N <= 8192 the workgroups of a wave cover whole
+    bands of 8 macro-tile rows, all XCDs working on the same A rows at the same time."""
+    hint = np.array(tiling.raster_hint(M, N, 1)).reshape(-1, 4)[:, 0]      # first layout tile of every workgroup
+    TN = N // 128
+    gm, gn = (hint // TN) // 2, (hint % TN) // 2
+    GN = N // 256
+    for w in range(len(hint) // 256):
+        rows = np.unique(gm[256 * w:256 * (w + 1)])
+        assert len(rows) * GN == 256 and rows.max() - rows.min() == len(rows) - 1
+        for r in rows:
+            assert sorted(gn[256 * w:256 * (w + 1)][gm[256 * w:256 * (w + 1)] == r]) == list(range(GN))
+
+
 def test_raster_hint_rejects_bad_shapes():
     with pytest.raises(capi.FoError):
         tiling.raster_hint(1000, 1024, 1)
