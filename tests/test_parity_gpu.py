@@ -424,6 +424,39 @@ def test_half_macro_tiles_scatter(L, dev):
     assert p.dMM.cpu()[:p.G].tolist() == cseg
 
 
+# ---- seeded random shapes ---------------------------------------------------------
+
+def _random_problem(seed):
+    """A shape the library accepts, drawn from a seed: any Algo, M and N multiples of its tile, K a
+    multiple of 8, a ragged partition of the tiles into groups and a random slot permutation."""
+    rng = np.random.default_rng(seed)
+    algo = int(rng.integers(0, 6))
+    BM, BN, _ = capi.algo_tile(algo)
+    M = BM * int(rng.integers(1, 2560 // BM + 1))
+    N = BN * int(rng.integers(1, 2560 // BN + 1))
+    K = 8 * int(rng.integers(1, 41))
+    T = (M // BM) * (N // BN)
+    cuts = sorted(rng.choice(np.arange(1, T), size=min(T - 1, int(rng.integers(0, 6))), replace=False).tolist()) if T > 1 else []
+    cseg = np.diff([0] + cuts + [T]).tolist()
+    return algo, M, N, K, T, cseg, rng.permutation(T).tolist()
+
+
+@pytest.mark.parametrize("seed", range(100, 116))
+def test_random_shapes_plain_and_signal_bit_exact(L, dev, seed):
+    algo, M, N, K, T, cseg, hint = _random_problem(seed)
+    dt = torch.float16 if seed % 2 else torch.bfloat16
+    _say("random shape", seed, dt, M, N, K, algo, cseg)
+    BM, BN, _ = capi.algo_tile(algo)
+    p = Path(L, dev, dt, M, N, K, algo, cseg=cseg, hint=hint, integer_inputs=True, seed=seed)
+    p.build_table()
+    want = O.gemm(p.A, p.B)
+    assert torch.equal(p.gemm_plain().cpu(), want)
+    p.gemm_signal(use_table=bool(seed & 2))
+    torch.cuda.synchronize()
+    assert torch.equal(p.dC.cpu(), O.place_tiles(want, p.ra_host.numpy(), BM, BN, 1))
+    assert p.dMM.cpu()[:p.G].tolist() == cseg and p.dMM.cpu()[p.G:].sum() == 0
+
+
 # ---- wait / consume ------------------------------------------------------------
 
 def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
