@@ -457,6 +457,22 @@ def test_random_shapes_plain_and_signal_bit_exact(L, dev, seed):
     assert p.dMM.cpu()[:p.G].tolist() == cseg and p.dMM.cpu()[p.G:].sum() == 0
 
 
+@pytest.mark.parametrize("seed", range(200, 208))
+def test_random_shapes_scatter_bit_exact(L, dev, seed):
+    algo, M, N, K, T, cseg, hint = _random_problem(seed)
+    ws = (2, 4, 8)[seed % 3]
+    _say("random scatter", seed, M, N, K, algo, ws, cseg)
+    BM, BN, _ = capi.algo_tile(algo)
+    p = Path(L, dev, torch.bfloat16, M, N, K, algo, cseg=cseg, hint=hint, ws=ws, integer_inputs=True, seed=seed)
+    assert p.re_host.tolist() == O.row_remap(M, N, BM, BN, cseg, ws).tolist()
+    p.build_table()
+    p.gemm_signal()
+    torch.cuda.synchronize()
+    want = O.scatter_place(O.gemm(p.A, p.B), p.ra_host.numpy(), p.re_host.numpy(), BM, BN, 1)
+    assert torch.equal(p.dC.cpu(), want)
+    assert p.dMM.cpu()[:p.G].tolist() == cseg
+
+
 # ---- wait / consume ------------------------------------------------------------
 
 def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
