@@ -81,6 +81,9 @@ struct Mma<_Float16> {
     static __device__ __forceinline__ void run(frag a, frag b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
+    static __device__ __forceinline__ void clear(frag zeros, f32x4& c) {   // c = 0 x 0 + 0
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %1, 0" : "=a"(c) : "v"(zeros));
+    }
 };
 template <>
 struct Mma<__bf16> {
@@ -88,6 +91,9 @@ struct Mma<__bf16> {
     using out4 = bf16x4;
     static __device__ __forceinline__ void run(frag a, frag b, f32x4& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void clear(frag zeros, f32x4& c) {   // c = 0 x 0 + 0
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %1, 0" : "=a"(c) : "v"(zeros));
     }
 };
 
@@ -313,13 +319,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) ko[h] = ((4 * h + fr_kc) ^ swz(fr_row)) * 16;
 
-    f32x4 acc[NB][NB];
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+    f32x4 acc[NB][NB];   // cleared in the prologue, while the first panels are on their way
 
     // Fragments of the two k halves of a panel.  Quarter step q works on k half
     // q/2 and on the A blocks (q%2)*NH .. +NH: its own A fragments and, in the
@@ -456,10 +456,21 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         issue_unit(1, 2 * PANEL, unit_a, second_half);
         issue_unit(1, 3 * PANEL, unit_b, first_half);
         issue_unit(1, 3 * PANEL, unit_b, second_half);
-        wait_vmcnt<LPT>();
-    } else {
-        wait_vmcnt<0>();
     }
+    // The accumulators are cleared here, under the latency of those copies, by MFMAs on zero
+    // operands (0 x 0 + 0).  Written as assignments of zero, the compiler places the 256 register
+    // writes directly in front of the main loop, behind the wait for the first panel.
+    {
+        frag zeros;
+        asm volatile("v_mov_b32 %0, 0\n\tv_mov_b32 %1, 0\n\tv_mov_b32 %2, 0\n\tv_mov_b32 %3, 0\n\ts_nop 7"
+                     : "=v"(((float*)&zeros)[0]), "=v"(((float*)&zeros)[1]), "=v"(((float*)&zeros)[2]),
+                       "=v"(((float*)&zeros)[3]));
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+#pragma unroll
+            for (int j = 0; j < NB; ++j) Mma<T>::clear(zeros, acc[i][j]);
+    }
+    if (NP > 1) wait_vmcnt<LPT>(); else wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     load_frags(0, PANEL, 0);
     wait_lds_reads();
