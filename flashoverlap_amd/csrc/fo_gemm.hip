@@ -129,7 +129,9 @@ struct GemmParams {
     void* D;
     int M, N, K;
     int GM, GN;   // macro-tile grid
+    unsigned gn_magic;   // raster_magic(GN)
     int BM, BN;   // layout tile
+    int log_bm, log_bn;   // both edges are powers of two (128 or 256): shifts instead of divisions in the kernel
     int TN;       // N / BN
     int rLDN;
     const int* RA;
@@ -203,7 +205,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
 
-    const TileCoord mt = raster_map(blockIdx.x, p.GM, p.GN);
+    const TileCoord mt = raster_map(blockIdx.x, p.GM, p.GN, p.gn_magic);
     const int K = p.K;
     // M and N are multiples of the layout tile, not necessarily of the macro
     // tile: the last row or column of macro tiles may be half inside.  Such a
@@ -215,39 +217,42 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 
     // ---- where this wavefront's quadrant goes -------------------------------
     // row0/col0/ld describe the destination of quadrant element (0,0) in a
-    // row-major view; rows are consecutive in that view (before RE).
-    int row0, col0, ld;
-    int sig_slot = 0, sig_group = 0;
-    if constexpr (MODE == kPlain) {
-        row0 = mt.m * MT + wm * WT;
-        col0 = mt.n * MT + wn * WT;
-        ld = p.N;
-    } else {
-        const int tiles_n = MT / p.BN;                // layout tiles per macro tile, N
-        const int tiles_m = MT / p.BM;
+    // row-major view; rows are consecutive in that view (before RE).  In the
+    // signalling modes they follow from the slot of the quadrant's layout tile.
+    // The slots (this wave's, and in the lanes that will signal that of "their"
+    // layout tile) are fetched here, ahead of the first panel copies, but looked at
+    // only behind the prologue's barrier, when they have long arrived: nothing may
+    // stand between the start of the kernel and the issue of those copies.  What
+    // depends on the slots (group, remapped rows) is fetched there too, under the
+    // first k-steps.
+    int row0 = mt.m * MT + wm * WT, col0 = mt.n * MT + wn * WT, ld = p.N;
+    int sig_slot = 0, sig_group = -1;   // -1: a lane without a layout tile inside the matrix stays out of the signal
+    [[maybe_unused]] int quad_slot = 0;
+    [[maybe_unused]] bool sig_lane = false;
+    if constexpr (MODE != kPlain) {
+        const int tiles_n = MT >> p.log_bn;           // layout tiles per macro tile, N
+        const int tiles_m = MT >> p.log_bm;
         const int qm = wm * WT, qn = wn * WT;         // quadrant origin in the macro tile
-        const int t = (mt.m * tiles_m + qm / p.BM) * p.TN + mt.n * tiles_n + qn / p.BN;
-        const int s = live ? __builtin_amdgcn_readfirstlane(p.RA[t]) : 0;
-        row0 = (s / p.rLDN) * p.BM + qm % p.BM;
-        col0 = (s % p.rLDN) * p.BN + qn % p.BN;
-        ld = p.rLDN * p.BN;
-        // The lanes that will signal look up their slot and group now, so the
-        // two dependent loads are hidden behind the main loop.
-        const int ntile = tiles_m * tiles_n;
-        sig_group = -1;   // lanes without a layout tile (or with one outside the matrix) stay out of the signal
-        if (tid < ntile && (tid / tiles_n) * p.BM < valid_m && (tid % tiles_n) * p.BN < valid_n) {
-            const int ts = (mt.m * tiles_m + tid / tiles_n) * p.TN + mt.n * tiles_n + tid % tiles_n;
-            sig_slot = p.RA[ts];
-            sig_group = p.gtable ? p.gtable[sig_slot] : scan_group(p.cseg, sig_slot);
+        if (live) quad_slot = p.RA[(mt.m * tiles_m + (qm >> p.log_bm)) * p.TN + mt.n * tiles_n + (qn >> p.log_bn)];
+        const int sig_m = tiles_n == 2 ? tid >> 1 : tid, sig_n = tiles_n == 2 ? tid & 1 : 0;   // tiles_n is 1 or 2
+        sig_lane = tid < tiles_m * tiles_n && (sig_m << p.log_bm) < valid_m && (sig_n << p.log_bn) < valid_n;
+        if (sig_lane) sig_slot = p.RA[(mt.m * tiles_m + sig_m) * p.TN + mt.n * tiles_n + sig_n];
+    }
+    [[maybe_unused]] int re_lo = 0, re_hi = 0;   // scatter: the remapped destination rows of this quadrant
+    auto resolve_destination = [&]() {
+        if constexpr (MODE != kPlain) {
+            const int s = __builtin_amdgcn_readfirstlane(quad_slot);
+            row0 = (s / p.rLDN) * p.BM + ((wm * WT) & (p.BM - 1));
+            col0 = (s % p.rLDN) * p.BN + ((wn * WT) & (p.BN - 1));
+            ld = p.rLDN * p.BN;
+            if (sig_lane) sig_group = p.gtable ? p.gtable[sig_slot] : scan_group(p.cseg, sig_slot);
         }
-    }
-    // Scatter: the remapped destination rows of this quadrant, one or two per
-    // lane, fetched now and handed round between the lanes in the epilogue.
-    [[maybe_unused]] int re_lo = 0, re_hi = 0;
-    if constexpr (MODE == kScatter) {
-        re_lo = p.RE[row0 + (lane < WT ? lane : 0)];
-        if constexpr (WT > 64) re_hi = p.RE[row0 + 64 + lane];
-    }
+        // Scatter: one or two remapped rows per lane, handed round between the lanes in the epilogue.
+        if constexpr (MODE == kScatter) {
+            re_lo = p.RE[row0 + (lane < WT ? lane : 0)];
+            if constexpr (WT > 64) re_hi = p.RE[row0 + 64 + lane];
+        }
+    };
 
     // ---- HBM -> LDS copy addressing ------------------------------------------
     // One copy instruction moves 1 KiB = 8 panel rows of 128 bytes: lane l's 16
@@ -473,6 +478,9 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     if (NP > 1) wait_vmcnt<LPT>(); else wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     load_frags(0, PANEL, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    resolve_destination();
+    __builtin_amdgcn_sched_barrier(0);
     wait_lds_reads();
 
     // The consumer's waves share SIMDs with these waves while a group is being
@@ -546,7 +554,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         // before the counter moves.
         wait_vmcnt<0>();
         __syncthreads();
-        const int ntile = (MT / p.BM) * (MT / p.BN);
+        const int ntile = (MT >> p.log_bm) * (MT >> p.log_bn);
         // The tiles of a macro tile mostly fall into one group: the first lane of
         // every distinct group adds that group's tile count in one atomic (at most
         // four lanes take part, all in the first wavefront).  Monitor mode keeps
@@ -634,6 +642,8 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
                 const int* RE, int monitor, hipStream_t stream) {
     int BM, BN, BK;
     if (algo_tile(algo, &BM, &BN, &BK) != FO_OK) return fail(FO_ERR_ARG, "fo_gemm: Algo %d out of range", algo);
+    if ((BM != 128 && BM != 256) || (BN != 128 && BN != 256))
+        return fail(FO_ERR_ARG, "fo_gemm: layout tile %dx%d: the kernel takes edges of 128 or 256", BM, BN);
     if (dtype != FO_F16 && dtype != FO_BF16) return fail(FO_ERR_ARG, "fo_gemm: dtype %d not fp16/bf16", dtype);
     if (!A || !B || !D) return fail(FO_ERR_ARG, "fo_gemm: null operand");
     if (M <= 0 || N <= 0 || K <= 0) return fail(FO_ERR_SHAPE, "fo_gemm: empty problem %dx%dx%d", M, N, K);
@@ -653,7 +663,9 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
     p.A = A; p.B = B; p.D = D;
     p.M = M; p.N = N; p.K = K;
     p.GM = (M + macro - 1) / macro; p.GN = (N + macro - 1) / macro;
+    p.gn_magic = raster_magic(p.GN);
     p.BM = BM; p.BN = BN; p.TN = N / BN;
+    p.log_bm = BM == 256 ? 8 : 7; p.log_bn = BN == 256 ? 8 : 7;
     p.rLDN = rLDN;
     p.RA = RA; p.RE = RE; p.cseg = cseg; p.G = G; p.gtable = gtable; p.MM = MM; p.monitor = monitor;
 
@@ -680,7 +692,7 @@ int raster_hint(int algo, int M, int N, int* hint) {
     const int tiles_m = macro / BM, tiles_n = macro / BN;
     int k = 0;
     for (int pid = 0; pid < GM * GN; ++pid) {
-        const TileCoord c = raster_map(pid, GM, GN);
+        const TileCoord c = raster_map(pid, GM, GN, raster_magic(GN));
         for (int i = 0; i < tiles_m; ++i)
             for (int j = 0; j < tiles_n; ++j) {
                 const int tm = c.m * tiles_m + i, tn = c.n * tiles_n + j;

@@ -28,8 +28,17 @@ struct TileCoord {
     int m, n;
 };
 
-// pid in [0, GM*GN) -> macro tile coordinate.
-FO_HD TileCoord raster_map(int pid, int GM, int GN) {
+// Division by the column count without a divide instruction (the kernel does this once per
+// workgroup, in front of its first memory access): n / d == (n * magic) >> 32 with
+// magic = 2^32 / d + 1, exact while n * d < 2^32 (tile counts are far below that).
+// (d = 1 has no such 32-bit magic; it is stored as 0.)
+FO_HD unsigned raster_magic(int d) { return d == 1 ? 0u : (unsigned)(0x100000000ull / (unsigned)d) + 1u; }
+FO_HD int raster_div(int n, unsigned magic) {
+    return magic ? (int)(((unsigned long long)(unsigned)n * magic) >> 32) : n;
+}
+
+// pid in [0, GM*GN) -> macro tile coordinate; gn_magic = raster_magic(GN).
+FO_HD TileCoord raster_map(int pid, int GM, int GN, unsigned gn_magic) {
     const int total = GM * GN;
     const int xcd = pid % kXcds, local = pid / kXcds;
     constexpr int kUnit = kGroupM * kUnitN, kWave = kXcds * kUnit;
@@ -39,16 +48,22 @@ FO_HD TileCoord raster_map(int pid, int GM, int GN) {
     const int pos = pid < whole ? ((local / kUnit) * kXcds + xcd) * kUnit + local % kUnit : pid;
     // Position -> tile: bands of kGroupM rows (the last may be lower), in a band blocks of kUnitN
     // columns (the last may be narrower), in a block column by column.
-    const int band_tiles = kGroupM * GN;
-    const int band = pos / band_tiles;
+    const int band = raster_div(pos / kGroupM, gn_magic);     // pos / (kGroupM * GN)
     const int first_m = band * kGroupM;
-    const int rows = (GM - first_m < kGroupM) ? (GM - first_m) : kGroupM;
-    const int in_band = pos - band * band_tiles;
-    const int block = in_band / (rows * kUnitN);
-    const int in_block = in_band - block * rows * kUnitN;
+    const int in_band = pos - band * kGroupM * GN;
     TileCoord c;
-    c.m = first_m + in_block % rows;
-    c.n = block * kUnitN + in_block / rows;
+    if (GM - first_m >= kGroupM) {                            // a full band: shifts only
+        const int block = in_band / (kGroupM * kUnitN);
+        const int in_block = in_band % (kGroupM * kUnitN);
+        c.m = first_m + in_block % kGroupM;
+        c.n = block * kUnitN + in_block / kGroupM;
+    } else {
+        const int rows = GM - first_m;
+        const int block = in_band / (rows * kUnitN);
+        const int in_block = in_band - block * rows * kUnitN;
+        c.m = first_m + in_block % rows;
+        c.n = block * kUnitN + in_block / rows;
+    }
     return c;
 }
 

@@ -70,7 +70,7 @@ def test_argument_errors_return_codes_not_exits(fo_lib):
 
 @pytest.mark.parametrize("algo,M,N", [(1, 1024, 1024), (1, 4096, 4096), (0, 8192, 4096), (1, 16384, 8192),
                                       (1, 8192, 8192), (3, 1024, 2048), (5, 2048, 1024), (1, 384, 640),
-                                      (1, 128, 128), (1, 2304, 256)])
+                                      (1, 128, 128), (1, 2304, 256), (3, 1152, 256), (1, 4480, 4224), (5, 256, 8320)])
 def test_raster_hint_is_a_permutation_grouped_by_workgroup(algo, M, N):
     BM, BN, _ = capi.algo_tile(algo)
     T = (M // BM) * (N // BN)
