@@ -512,12 +512,15 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     __syncthreads();  // every wave is done with the panel buffers
     constexpr int PITCH = WT * 2 + 16;                  // strip row pitch in bytes
     constexpr int ROWCH = WT / 8;                       // 16-byte chunks per strip row
-    unsigned char* ep = smem + wave * (32 * PITCH);
+    // Two strip buffers per wave, used in turn: the next strip is written while this one is being stored.
+    unsigned char* ep0 = smem + wave * (32 * PITCH);
+    unsigned char* ep1 = ep0 + 4 * 32 * PITCH;
     T* D = (T*)p.D;
     [[maybe_unused]] __amdgpu_buffer_rsrc_t drsrc;
     if constexpr (STORE == 1) drsrc = __builtin_amdgcn_make_buffer_rsrc(p.D, 0, 0xffffffff, 0x00020000);
 #pragma unroll
     for (int i = 0; i < NB / 2; ++i) {   // strip i: rows 32i .. 32i+31 of the quadrant
+        unsigned char* ep = (i & 1) ? ep1 : ep0;
 #pragma unroll
         for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
@@ -588,7 +591,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 template <typename T, int MT, int MODE, int STORE, int REL>
 static int launch_one(const GemmParams& p, hipStream_t stream) {
     constexpr int smem_bytes = 5 * MT * kRowBytes;   // five panel slots: 160 KiB at MT = 256
-    static_assert(4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the panel slots");
+    static_assert(2 * 4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the panel slots");
     auto kern = gemm_kernel<T, MT, MODE, STORE, REL>;
     // The attribute belongs to the function on one device: set it once per device.
     static std::atomic<unsigned long long> configured{0};
