@@ -102,6 +102,8 @@ def main() -> int:
                     help="c2/c4: also time the step under the other reading and put it into the record")
     ap.add_argument("--kernel-iters", type=int, default=100, help="timed launches per isolated kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline work; 0 skips it")
+    ap.add_argument("--mfma-loop-seconds", type=float, default=0.6,
+                    help="how long to run the MFMA-only loop (fo_mfma_spin) on each operand set; 0 skips it")
     ap.add_argument("--consumer-blocks", type=int, default=0,
                     help="workgroups of the persistent consumer (0 = one per CU, which is also the maximum)")
     ap.add_argument("--consumer", default="auto", choices=["auto", "per_group", "persistent"])
@@ -348,7 +350,6 @@ def main() -> int:
     # the power limit, not the kernel's schedule.
     A0, B0 = torch.zeros_like(A), torch.zeros_like(B)
     z_ms, _ = time_kernel(lambda i: gemm_plain(A0, B0), max(10, it // 4))
-    del A0, B0
 
     other = None
     if a.both_readings and a.workload in WAVE_READING and not a.group_tiles:
@@ -364,6 +365,32 @@ def main() -> int:
                  "consumer": consumer_name(g2), "ms_per_step": round(s2_ms, 5), "serial_step_ms": round(s2_serial, 5),
                  "gemm_signal_in_step_us": round(s2_gemm * 1e3, 2), "gemm_signal_isolated_us": round(sig2_ms * 1e3, 2),
                  "signal_overhead_pct": round((sig2_ms / pl_ms - 1.0) * 100.0, 2)}
+
+    # What the power limit leaves to the MFMAs alone: the GEMM's own MFMA instruction in a loop on
+    # register operands taken from A (and from zeros), no memory, LDS or address work beside it.
+    # The GEMM's rate can be read against the first figure: no kernel on these operands gets past it.
+    mfma_loop = None
+    if a.mfma_loop_seconds > 0:
+        sink = torch.zeros(1, dtype=torch.float32, device=dev)
+        spin_flop = C.c_longlong()
+
+        def spin_rate(buf, wide=0):
+            def launch(i):      # 2048 rounds of 64 MFMAs per wavefront: about 1 ms
+                capi.check(L.fo_mfma_spin(code, wide, buf.data_ptr(), buf.numel() * buf.element_size(), 2048,
+                                          sink.data_ptr(), C.byref(spin_flop), main_stream))
+            n = max(8, int(a.mfma_loop_seconds / 2 / 1e-3))
+            for i in range(n):  # first half untimed: the clock settles to what the power limit allows
+                launch(i)
+            ms, _ = time_kernel(launch, n)
+            tf = spin_flop.value / ms / 1e9
+            return {"achieved": round(tf, 1), "frac": round(tf / PEAK_MFMA_TFLOPS, 4), "avg_us": round(ms * 1e3, 2)}
+
+        mfma_loop = {"unit": "TFLOP/s", "instruction": f"v_mfma_f32_16x16x32_{'f16' if dts == 'fp16' else 'bf16'}",
+                     "operands_of_A": spin_rate(A), "zero_operands": spin_rate(A0),
+                     "operands_of_A_32x32x16": spin_rate(A, 1),
+                     "note": "one wavefront per SIMD issuing nothing but MFMAs on register operands, sustained "
+                             f"{a.mfma_loop_seconds / 2:.1f} s before the timed half"}
+    del A0, B0
 
     flops = 2.0 * M * N * K
     rms_bytes = 2.0 * (M * N * 2) + N * 2
@@ -425,20 +452,21 @@ def main() -> int:
         # the same kernel launched back to back on its own (A and B stay in the 256 MB memory-side cache)
         "gemm_signal_isolated": {"achieved": round(sig_tf, 2), "unit": "TFLOP/s",
                                  "frac": round(sig_tf / PEAK_MFMA_TFLOPS, 4), "avg_us": round(sig_ms * 1e3, 2),
-                                 "min_us": round(sig_min * 1e3, 2), "launches": it},
+                                 "min_single_launch_us": round(sig_min * 1e3, 2), "launches": it},
         "cpu_baseline": cpu,
         "gemm_plain": {"achieved": round(pl_tf, 2), "unit": "TFLOP/s", "frac": round(pl_tf / PEAK_MFMA_TFLOPS, 4),
-                       "avg_us": round(pl_ms * 1e3, 2), "min_us": round(pl_min * 1e3, 2)},
+                       "avg_us": round(pl_ms * 1e3, 2), "min_single_launch_us": round(pl_min * 1e3, 2)},
         "gemm_plain_zero_operands": {"achieved": round(flops / z_ms / 1e9, 2), "unit": "TFLOP/s",
                                      "frac": round(flops / z_ms / 1e9 / PEAK_MFMA_TFLOPS, 4),
                                      "avg_us": round(z_ms * 1e3, 2),
                                      "note": "same kernel and shape, A = B = 0: not power-limited"},
+        "mfma_only_loop": mfma_loop,
         "signal_overhead_pct": round((sig_ms / pl_ms - 1.0) * 100.0, 2),
         # headline: back to back over a rotation of buffer pairs that exceeds the memory-side cache
         "reorder_rmsnorm": {"bound": "hbm", "peak": PEAK_HBM_GBPS, "unit": "GB/s", "bytes": rms_bytes,
                             **hbm(rms_rot_ms), "buffer_pairs": npairs,
                             "in_step": hbm(step_norm_ms),
-                            "same_pair_back_to_back": {**hbm(rms_same_ms), "min_us": round(rms_min * 1e3, 2)}},
+                            "same_pair_back_to_back": {**hbm(rms_same_ms), "min_single_launch_us": round(rms_min * 1e3, 2)}},
         "consume_copy": {"achieved": round(cons_bytes / cons_ms / 1e6, 1), "unit": "GB/s",
                          "avg_us": round(cons_ms * 1e3, 2)},
         "other_reading": other,

@@ -21,7 +21,7 @@ LIB = os.path.join(HERE, "lib")
 OBJ = os.path.join(HERE, "build")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["fo_capi.hip", "fo_gemm.hip", "fo_sync.hip", "fo_rmsnorm.hip", "fo_static.hip"]
+HIP_SOURCES = ["fo_capi.hip", "fo_gemm.hip", "fo_sync.hip", "fo_rmsnorm.hip", "fo_static.hip", "fo_probe.hip"]
 BINDING_SOURCES = ["overlap_impl.cpp", "baseline_impl.cpp", "rmsnorm_op.cpp", "pybind.cpp"]
 
 # -packed-fp32-ops: keep hipcc from forming packed-fp32 instructions out of scalar float code.

@@ -193,6 +193,42 @@ def test_time_next_launch_gives_the_kernel_duration(L, dev):
         capi.check(L.fo_event_destroy(e))
 
 
+@pytest.mark.parametrize("wide", [0, 1])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wide):
+    """The MFMA-only loop used as the power-limit yardstick: reads its operands inside the buffer
+    it is given (an odd number of 16-byte chunks here), reports 64 MFMAs x 16384 flop (or 32 x
+    32768) x 4 wavefronts x CUs per round, writes nothing, and is not faster than the chip."""
+    cu = C.c_int()
+    capi.check(L.fo_device_info(C.byref(cu), None, None))
+    buf = torch.randn(7 * 8, device=dev).to(dt)            # 7 chunks of 16 bytes
+    guard = torch.full((64,), 3.0, dtype=torch.float32, device=dev)
+    flop = C.c_longlong()
+    iters = 2048
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    capi.check(L.fo_event_create(C.byref(e0)))
+    capi.check(L.fo_event_create(C.byref(e1)))
+    args = (capi.dtype_code(dt), wide, buf.data_ptr(), buf.numel() * 2, iters, guard[32:].data_ptr(), C.byref(flop), None)
+    capi.check(L.fo_mfma_spin(*args))
+    capi.check(L.fo_event_record(e0, None))
+    capi.check(L.fo_mfma_spin(*args))
+    capi.check(L.fo_event_record(e1, None))
+    torch.cuda.synchronize()
+    ms = C.c_float()
+    capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(ms)))
+    assert flop.value == cu.value * 4 * iters * 64 * 2 * 16 * 16 * 32
+    assert torch.equal(guard.cpu(), torch.full((64,), 3.0))
+    rate = flop.value / (ms.value * 1e-3)
+    _say("  MFMA-only loop %.0f TFLOP/s" % (rate / 1e12))
+    assert 0.3e15 < rate < 2.6e15
+    assert L.fo_mfma_spin(7, *args[1:]) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], wide, None, 16, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], wide, buf.data_ptr(), 8, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], wide, buf.data_ptr(), 112, 0, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    capi.check(L.fo_event_destroy(e0))
+    capi.check(L.fo_event_destroy(e1))
+
+
 def test_gemm_rejects_unsupported_shapes(L, dev):
     a = torch.zeros(384, 384, dtype=torch.float16, device=dev)  # large enough for every call below
     assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 44, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
