@@ -396,7 +396,10 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
                 copier(template_int<(sl - cstart) / 2>{});
             __builtin_amdgcn_sched_barrier(0);
             // operands swapped (B rows as the MFMA "A" matrix): a lane ends up with 4 consecutive n for one m
-            Mma<T>::run(fb[h][sl % NB], fa[h][i0 + sl / NB], acc[i0 + sl / NB][sl % NB]);
+            // Rows of blocks are walked back and forth, so that exactly one of the two operands changes
+            // from one MFMA to the next: an operand change costs power, and power is what limits this kernel.
+            constexpr int mi = i0 + sl / NB, mj = ((sl / NB) & 1) ? NB - 1 - sl % NB : sl % NB;
+            Mma<T>::run(fb[h][mj], fa[h][mi], acc[mi][mj]);
             __builtin_amdgcn_sched_barrier(0);
         });
     };
