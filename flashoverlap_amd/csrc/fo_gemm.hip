@@ -379,7 +379,8 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         constexpr int i0 = hs * NH;
         static_for<NS>([&](auto s_c) {
             constexpr int sl = decltype(s_c)::value;
-            constexpr int j = sl / COL, w = sl % COL, r = w / 2, h = w & 1;
+            constexpr int j = sl / COL, w = sl % COL, h = w & 1;
+            constexpr int r = (j & 1) ? NH - 1 - w / 2 : w / 2;   // rows down one column, up the next: the A pair stays over the turn
             if constexpr (hs == 0) {
                 if constexpr (w == 0) {
                     constexpr int own = 2 * (j < NH ? j : NH);

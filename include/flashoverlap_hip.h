@@ -271,15 +271,15 @@ int fo_stream_is_capturing(void* stream, int* capturing);
 
 /* Measurement aid, no counterpart in the reference: one launch of a kernel that does nothing but
  * the GEMM's MFMA instruction (v_mfma_f32_16x16x32 of `dtype`) on operands held in registers:
- * one workgroup of 4 wavefronts per CU, 64 independent accumulators per wavefront, `iters`
- * rounds of 64 MFMAs each (wide != 0: v_mfma_f32_32x32x16 instead, 16 accumulators, 32 MFMAs a
- * round, the same flop).  Every lane reads its 16 operand fragments (16 bytes each) once from
- * `operands` (any device buffer of operand_bytes >= 16 bytes, read modulo its size): pass the
- * GEMM's own A or B and the loop toggles the matrix cores like the GEMM does, pass zeros and it
- * toggles nothing.  The GEMM runs at the chip's power limit, so the rate of this loop on the same
- * operands, not the clock-times-width peak, is what the hardware leaves for it to reach.
- * `sink` (>= 4 bytes of device memory) is never written in practice; *flop, if not null, receives
- * the floating-point operations of the launch. */
+ * one workgroup of 4 wavefronts per CU, 8 x 8 accumulators per wavefront, `iters` rounds of 128
+ * MFMAs each in the order of the GEMM's k-step (wide != 0: v_mfma_f32_32x32x16 instead, 4 x 4
+ * accumulators, 64 MFMAs a round, the same flop).  Every lane reads its 32 operand fragments (16
+ * bytes each) once from `operands` (any device buffer of operand_bytes >= 16 bytes, read modulo
+ * its size): pass the GEMM's own A or B and the loop toggles the matrix cores like the GEMM does,
+ * pass zeros and it toggles nothing.  The GEMM runs at the chip's power limit, so the rate of
+ * this loop on the same operands, not the clock-times-width peak, is what the hardware leaves
+ * for it to reach.  `sink` (>= 4 bytes of device memory) is never written in practice; *flop, if
+ * not null, receives the floating-point operations of the launch. */
 int fo_mfma_spin(int dtype, int wide, const void* operands, size_t operand_bytes, int iters, void* sink,
                  long long* flop, void* stream);
 

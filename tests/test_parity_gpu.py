@@ -197,14 +197,14 @@ def test_time_next_launch_gives_the_kernel_duration(L, dev):
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wide):
     """The MFMA-only loop used as the power-limit yardstick: reads its operands inside the buffer
-    it is given (an odd number of 16-byte chunks here), reports 64 MFMAs x 16384 flop (or 32 x
+    it is given (an odd number of 16-byte chunks here), reports 128 MFMAs x 16384 flop (or 64 x
     32768) x 4 wavefronts x CUs per round, writes nothing, and is not faster than the chip."""
     cu = C.c_int()
     capi.check(L.fo_device_info(C.byref(cu), None, None))
     buf = torch.randn(7 * 8, device=dev).to(dt)            # 7 chunks of 16 bytes
     guard = torch.full((64,), 3.0, dtype=torch.float32, device=dev)
     flop = C.c_longlong()
-    iters = 2048
+    iters = 1024
     e0, e1 = C.c_void_p(), C.c_void_p()
     capi.check(L.fo_event_create(C.byref(e0)))
     capi.check(L.fo_event_create(C.byref(e1)))
@@ -216,7 +216,7 @@ def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wi
     torch.cuda.synchronize()
     ms = C.c_float()
     capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(ms)))
-    assert flop.value == cu.value * 4 * iters * 64 * 2 * 16 * 16 * 32
+    assert flop.value == cu.value * 4 * iters * 128 * 2 * 16 * 16 * 32
     assert torch.equal(guard.cpu(), torch.full((64,), 3.0))
     rate = flop.value / (ms.value * 1e-3)
     _say("  MFMA-only loop %.0f TFLOP/s" % (rate / 1e12))
