@@ -374,9 +374,9 @@ def main() -> int:
         sink = torch.zeros(1, dtype=torch.float32, device=dev)
         spin_flop = C.c_longlong()
 
-        def spin_rate(buf, wide=0):
+        def spin_rate(buf, wide=0, traffic=0):
             def launch(i):      # 1024 rounds of 128 MFMAs per wavefront: about 1 ms
-                capi.check(L.fo_mfma_spin(code, wide, buf.data_ptr(), buf.numel() * buf.element_size(), 1024,
+                capi.check(L.fo_mfma_spin(code, wide, traffic, buf.data_ptr(), buf.numel() * buf.element_size(), 1024,
                                           sink.data_ptr(), C.byref(spin_flop), main_stream))
             n = max(8, int(a.mfma_loop_seconds / 2 / 1e-3))
             for i in range(n):  # first half untimed: the clock settles to what the power limit allows
@@ -388,6 +388,10 @@ def main() -> int:
         mfma_loop = {"unit": "TFLOP/s", "instruction": f"v_mfma_f32_16x16x32_{'f16' if dts == 'fp16' else 'bf16'}",
                      "operands_of_A": spin_rate(A), "zero_operands": spin_rate(A0),
                      "operands_of_A_32x32x16": spin_rate(A, 1),
+                     # the same loop with the fragment reads and the copies of a 256x256 tile beside the MFMAs,
+                     # nothing waiting for them: this tile's operand traffic under a perfect schedule
+                     "operands_of_A_with_fragment_reads": spin_rate(A, 0, 1),
+                     "operands_of_A_with_tile_traffic": spin_rate(A, 0, 3),
                      "note": "one wavefront per SIMD issuing nothing but MFMAs on register operands, in the order of the GEMM's k-step, sustained "
                              f"{a.mfma_loop_seconds / 2:.1f} s before the timed half"}
     del A0, B0

@@ -47,7 +47,7 @@ SIGNATURES = {
     "fo_stream_join": (_i, [_vp, _vp]),
     "fo_stream_is_capturing": (_i, [_vp, C.POINTER(C.c_int)]),
     "fo_time_next_launch": (_i, [_vp, _vp]),
-    "fo_mfma_spin": (_i, [_i, _i, _vp, _sz, _i, _vp, C.POINTER(_ll), _vp]),
+    "fo_mfma_spin": (_i, [_i, _i, _i, _vp, _sz, _i, _vp, C.POINTER(_ll), _vp]),
     "fo_event_create": (_i, [C.POINTER(_vp)]),
     "fo_event_destroy": (_i, [_vp]),
     "fo_event_record": (_i, [_vp, _vp]),

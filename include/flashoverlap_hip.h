@@ -278,10 +278,15 @@ int fo_stream_is_capturing(void* stream, int* capturing);
  * its size): pass the GEMM's own A or B and the loop toggles the matrix cores like the GEMM does,
  * pass zeros and it toggles nothing.  The GEMM runs at the chip's power limit, so the rate of
  * this loop on the same operands, not the clock-times-width peak, is what the hardware leaves
- * for it to reach.  `sink` (>= 4 bytes of device memory) is never written in practice; *flop, if
- * not null, receives the floating-point operations of the launch. */
-int fo_mfma_spin(int dtype, int wide, const void* operands, size_t operand_bytes, int iters, void* sink,
-                 long long* flop, void* stream);
+ * for it to reach.  `traffic` adds, beside the MFMAs and with nothing waiting for it, what the
+ * GEMM's 256x256 tile moves per k-step and wavefront: bit 0 its 32 fragment reads (LDS to
+ * registers), bit 1 its 16 one-KiB copies (L2 to LDS; needs 4 MiB..4 GiB of operands, of which a
+ * power-of-two window is walked, four workgroups per XCD sharing a stream like the GEMM's tiles
+ * share panels); 3 is the GEMM's whole operand traffic under a perfect schedule; wide must then be
+ * 0.  `sink` (>= 4 bytes of device memory) is never written in practice; *flop, if not null,
+ * receives the floating-point operations of the launch. */
+int fo_mfma_spin(int dtype, int wide, int traffic, const void* operands, size_t operand_bytes, int iters,
+                 void* sink, long long* flop, void* stream);
 
 /* Timing helpers for harnesses that cannot use torch events on foreign
  * streams: opaque hipEvent_t handles. */

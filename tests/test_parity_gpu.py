@@ -193,22 +193,26 @@ def test_time_next_launch_gives_the_kernel_duration(L, dev):
         capi.check(L.fo_event_destroy(e))
 
 
-@pytest.mark.parametrize("wide", [0, 1])
+@pytest.mark.parametrize("wide,traffic", [(0, 0), (1, 0), (0, 1), (0, 2), (0, 3)])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
-def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wide):
-    """The MFMA-only loop used as the power-limit yardstick: reads its operands inside the buffer
-    it is given (an odd number of 16-byte chunks here), reports 128 MFMAs x 16384 flop (or 64 x
-    32768) x 4 wavefronts x CUs per round, writes nothing, and is not faster than the chip."""
+def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wide, traffic):
+    """The MFMA-only loop used as the power-limit yardstick, bare and with a GEMM tile's fragment
+    reads and copies beside it: reads its operands inside the buffer it is given (an odd number
+    of 16-byte chunks where it makes no copies, 4 MiB + 16 bytes where it does), reports 128 MFMAs
+    x 16384 flop (or 64 x 32768) x 4 wavefronts x CUs per round, writes nothing outside its own
+    LDS, and is not faster than the chip."""
     cu = C.c_int()
     capi.check(L.fo_device_info(C.byref(cu), None, None))
-    buf = torch.randn(7 * 8, device=dev).to(dt)            # 7 chunks of 16 bytes
+    nelem = (4 << 20) // 2 + 8 if traffic & 2 else 7 * 8
+    buf = torch.randn(nelem + 64, device=dev).to(dt)
+    tail = buf[nelem:].clone()                               # what lies behind the bytes handed over
     guard = torch.full((64,), 3.0, dtype=torch.float32, device=dev)
     flop = C.c_longlong()
     iters = 1024
     e0, e1 = C.c_void_p(), C.c_void_p()
     capi.check(L.fo_event_create(C.byref(e0)))
     capi.check(L.fo_event_create(C.byref(e1)))
-    args = (capi.dtype_code(dt), wide, buf.data_ptr(), buf.numel() * 2, iters, guard[32:].data_ptr(), C.byref(flop), None)
+    args = (capi.dtype_code(dt), wide, traffic, buf.data_ptr(), nelem * 2, iters, guard[32:].data_ptr(), C.byref(flop), None)
     capi.check(L.fo_mfma_spin(*args))
     capi.check(L.fo_event_record(e0, None))
     capi.check(L.fo_mfma_spin(*args))
@@ -218,13 +222,17 @@ def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wi
     capi.check(L.fo_event_elapsed_ms(e0, e1, C.byref(ms)))
     assert flop.value == cu.value * 4 * iters * 128 * 2 * 16 * 16 * 32
     assert torch.equal(guard.cpu(), torch.full((64,), 3.0))
+    assert torch.equal(buf[nelem:], tail)
     rate = flop.value / (ms.value * 1e-3)
-    _say("  MFMA-only loop %.0f TFLOP/s" % (rate / 1e12))
+    _say("  MFMA loop, wide %d traffic %d: %.0f TFLOP/s" % (wide, traffic, rate / 1e12))
     assert 0.3e15 < rate < 2.6e15
     assert L.fo_mfma_spin(7, *args[1:]) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], wide, None, 16, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], wide, buf.data_ptr(), 8, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], wide, buf.data_ptr(), 112, 0, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], wide, 4, *args[3:]) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], 1, 1, *args[3:]) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], 0, 2, buf.data_ptr(), 1 << 20, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], wide, 0, None, 16, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], wide, 0, buf.data_ptr(), 8, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert L.fo_mfma_spin(args[0], wide, 0, buf.data_ptr(), 112, 0, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
     capi.check(L.fo_event_destroy(e0))
     capi.check(L.fo_event_destroy(e1))
 
