@@ -22,17 +22,21 @@
 // this tile size the kernel sits at the edge of that request rate, so half-line
 // requests cost a quarter of the throughput.  The 16-byte chunks of a row are
 // XOR-swizzled by row so the ds_read_b128 fragment reads are bank-conflict
-// free.  A k-step of 64 is four quarter steps of 32 MFMAs each (two per k half
-// of 32); the fragments of all four are read during the first two, so while
-// one quarter's MFMAs run the fragments of the next are already in registers,
-// and the workgroup
-// barrier that releases the panel's two slots sits in the middle of the
-// k-step.  The free slot lets the copies of A(p+2) go out in the first half of
-// k-step p and those of B(p+2) in the second half: the same number of copies
-// in every quarter step, and between one and three more quarter steps for
-// them to land than with two buffers, which is what the kernel needs when its
-// operands come from HBM and not from the memory-side cache.  There is one
-// barrier per k-step.
+// free.  A k-step of 64 is two half steps of 64 MFMAs, each over half the rows
+// of blocks and walked column by column, with the two MFMAs that an
+// accumulator gets from the panel (k halves 0 and 1) issued back to back: the
+// second then takes the running sum from inside the matrix core instead of
+// from the register file, which lowers the power per flop and with it raises
+// the clock the power limit allows.  All B fragments of the panel stay in
+// registers for the whole k-step and are replaced, column by column, by those
+// of the next panel during the second half step; the A fragments of the
+// second half step are read during the first, so all reads of a panel are out
+// by the middle of its k-step, where the workgroup barrier that releases the
+// panel's two slots sits.  The free slot lets the copies of A(p+2) go out in
+// the first half of k-step p and those of B(p+2) in the second half, one
+// every few MFMAs, with more than a k-step to land, which is what the kernel
+// needs when its operands come from HBM and not from the memory-side cache.
+// There is one barrier per k-step.
 //
 // Epilogue: the quadrant goes through LDS in strips of 32 rows so that every
 // global store instruction writes four whole 256-byte row segments, either to
@@ -189,7 +193,7 @@ template <typename T, int MT, int MODE, int STORE, int REL>
 __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     constexpr int WT = MT / 2;               // wave quadrant edge
     constexpr int NB = WT / 16;              // 16x16 MFMA blocks per quadrant edge
-    constexpr int NH = NB / 2;               // A blocks per quarter step
+    constexpr int NH = NB / 2;               // rows of blocks per half step
     constexpr int PANEL = MT * kRowBytes;    // bytes of one A (or B) panel = one LDS slot
     constexpr int LOADS = MT / 32;           // wave-wide 1 KiB copies per wave per panel
     constexpr int LPT = 2 * LOADS;           // copies per wave per k-step
