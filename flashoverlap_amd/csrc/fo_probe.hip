@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void mfma_spin_kernel(const uint4* __restrict_
         for (int i = 0; i < 8; ++i) land[i] = a[0][i % F];
     }
     [[maybe_unused]] const unsigned rd =
-        (unsigned)(size_t)(lds) + (wave * 16 + (l & 15)) * 128 + (((((l >> 4) & 1) * 2 + (l >> 5)) ^ (l & 7)) * 16);
+        (unsigned)(__UINTPTR_TYPE__)((spin_lds_void*)lds) + (wave * 16 + (l & 15)) * 128 + (((((l >> 4) & 1) * 2 + (l >> 5)) ^ (l & 7)) * 16);
     [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc;
     [[maybe_unused]] unsigned goff = 0;
     if constexpr ((TRAFFIC & 2) != 0) {
