@@ -376,13 +376,14 @@ def main() -> int:
     # The GEMM's rate can be read against the first figure: no kernel on these operands gets past it.
     mfma_loop = None
     if a.mfma_loop_seconds > 0:
+        LB = capi.bench_lib()   # the probes live in a library of their own, outside the product's ABI
         sink = torch.zeros(1, dtype=torch.float32, device=dev)
         spin_flop = C.c_longlong()
 
         def spin_rate(buf, wide=0, traffic=0):
             def launch(i):      # 1024 rounds of 128 MFMAs per wavefront: about 1 ms
-                capi.check(L.fo_mfma_spin(code, wide, traffic, buf.data_ptr(), buf.numel() * buf.element_size(), 1024,
-                                          sink.data_ptr(), C.byref(spin_flop), main_stream))
+                capi.bench_check(LB.fo_mfma_spin(code, wide, traffic, buf.data_ptr(), buf.numel() * buf.element_size(),
+                                                 1024, sink.data_ptr(), C.byref(spin_flop), main_stream))
             n = max(8, int(a.mfma_loop_seconds / 2 / 1e-3))
             for i in range(n):  # first half untimed: the clock settles to what the power limit allows
                 launch(i)

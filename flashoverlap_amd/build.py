@@ -3,8 +3,10 @@
   flashoverlap_amd/lib/libfo_hip.so        HIP kernels + the C ABI (hipcc)
   flashoverlap_amd/lib/libst_pybinding.so  OverlapImpl / BaselineImpl / ops (g++ + torch headers),
                                            linked against libfo_hip.so only through the C ABI
+  flashoverlap_amd/lib/libfo_bench.so      measurement probes that only bench.py and its test load
+                                           (include/flashoverlap_bench.h); not part of the product
 
-Usage: python -m flashoverlap_amd.build [--only hip|binding] [-j N]
+Usage: python -m flashoverlap_amd.build [--only hip|binding|bench] [-j N]
 hipcc cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is.
 """
 from __future__ import annotations
@@ -21,7 +23,8 @@ LIB = os.path.join(HERE, "lib")
 OBJ = os.path.join(HERE, "build")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["fo_capi.hip", "fo_gemm.hip", "fo_sync.hip", "fo_rmsnorm.hip", "fo_static.hip", "fo_probe.hip"]
+HIP_SOURCES = ["fo_capi.hip", "fo_gemm.hip", "fo_sync.hip", "fo_rmsnorm.hip", "fo_static.hip"]
+BENCH_SOURCES = ["fo_probe.hip"]
 BINDING_SOURCES = ["overlap_impl.cpp", "baseline_impl.cpp", "rmsnorm_op.cpp", "pybind.cpp"]
 
 # -packed-fp32-ops: keep hipcc from forming packed-fp32 instructions out of scalar float code.
@@ -40,17 +43,25 @@ def _run(cmd):
         print(out)
 
 
-def build_hip(jobs: int = 4) -> str:
+def _build_hip_library(sources, name: str, jobs: int) -> str:
     os.makedirs(LIB, exist_ok=True)
     os.makedirs(OBJ, exist_ok=True)
     hipcc = os.path.join(ROCM, "bin", "hipcc")
-    objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in HIP_SOURCES]
-    cmds = [[hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(HIP_SOURCES, objs)]
+    objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in sources]
+    cmds = [[hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(sources, objs)]
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(_run, cmds))
-    out = os.path.join(LIB, "libfo_hip.so")
+    out = os.path.join(LIB, name)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out])
     return out
+
+
+def build_hip(jobs: int = 4) -> str:
+    return _build_hip_library(HIP_SOURCES, "libfo_hip.so", jobs)
+
+
+def build_bench(jobs: int = 4) -> str:
+    return _build_hip_library(BENCH_SOURCES, "libfo_bench.so", jobs)
 
 
 def build_binding(jobs: int = 4) -> str:
@@ -77,15 +88,18 @@ def build_binding(jobs: int = 4) -> str:
 def build_all(jobs: int = 4) -> None:
     build_hip(jobs)
     build_binding(jobs)
+    build_bench(jobs)
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", choices=["hip", "binding"])
+    ap.add_argument("--only", choices=["hip", "binding", "bench"])
     ap.add_argument("-j", type=int, default=4)
     a = ap.parse_args()
     if a.only in (None, "hip"):
         print(build_hip(a.j))
     if a.only in (None, "binding"):
         print(build_binding(a.j))
+    if a.only in (None, "bench"):
+        print(build_bench(a.j))
     sys.exit(0)

@@ -47,7 +47,6 @@ SIGNATURES = {
     "fo_stream_join": (_i, [_vp, _vp]),
     "fo_stream_is_capturing": (_i, [_vp, C.POINTER(C.c_int)]),
     "fo_time_next_launch": (_i, [_vp, _vp]),
-    "fo_mfma_spin": (_i, [_i, _i, _i, _vp, _sz, _i, _vp, C.POINTER(_ll), _vp]),
     "fo_event_create": (_i, [C.POINTER(_vp)]),
     "fo_event_destroy": (_i, [_vp]),
     "fo_event_record": (_i, [_vp, _vp]),
@@ -55,7 +54,15 @@ SIGNATURES = {
     "fo_event_elapsed_ms": (_i, [_vp, _vp, C.POINTER(_f)]),
 }
 
+# libfo_bench.so (include/flashoverlap_bench.h): measurement probes, loaded by bench.py and its test only.
+BENCH_LIB_PATH = os.path.join(_HERE, "lib", "libfo_bench.so")
+BENCH_SIGNATURES = {
+    "fo_bench_last_error": (C.c_char_p, []),
+    "fo_mfma_spin": (_i, [_i, _i, _i, _vp, _sz, _i, _vp, C.POINTER(_ll), _vp]),
+}
+
 _lib = None
+_bench_lib = None
 
 
 class FoError(RuntimeError):
@@ -85,6 +92,29 @@ def lib() -> C.CDLL:
             key, _, value = item.partition("=")
             check(handle.fo_tune(key.strip().encode(), int(value)))
     return _lib
+
+
+def bench_lib() -> C.CDLL:
+    """The measurement-probe library with argtypes set; raises if it is not built."""
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise FileNotFoundError(f"{BENCH_LIB_PATH} is missing: build it with `python -m flashoverlap_amd.build`")
+        try:
+            import torch  # noqa: F401
+        except Exception:
+            pass
+        handle = C.CDLL(BENCH_LIB_PATH, mode=C.RTLD_LOCAL)
+        for name, (res, args) in BENCH_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _bench_lib = handle
+    return _bench_lib
+
+
+def bench_check(code: int) -> None:
+    if code != FO_OK:
+        raise FoError(code, bench_lib().fo_bench_last_error().decode())
 
 
 def check(code: int) -> None:

@@ -14,12 +14,28 @@
 // wavefront, bit 1 its 16 one-KiB copies (L2 -> LDS, four workgroups per XCD reading the same
 // stream, so three in four hit the L2 as in the GEMM).  The rate with both is what the power limit
 // leaves to a kernel with this tile's operand traffic and a perfect schedule.
-// No counterpart in the reference.
+// No counterpart in the reference.  Built into libfo_bench.so, a library of its own that only the
+// benchmark and its test load: nothing here is part of the product's C ABI.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
 #include <type_traits>
 
-#include "fo_internal.h"
+#include "../../include/flashoverlap_bench.h"
 
 namespace fo {
+
+static thread_local char t_bench_error[256] = "";
+
+static int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+static int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(t_bench_error, sizeof t_bench_error, fmt, ap);
+    va_end(ap);
+    return code;
+}
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
@@ -136,6 +152,8 @@ __global__ __launch_bounds__(256) void mfma_spin_kernel(const uint4* __restrict_
 
 }  // namespace fo
 
+extern "C" const char* fo_bench_last_error(void) { return fo::t_bench_error; }
+
 extern "C" int fo_mfma_spin(int dtype, int wide, int traffic, const void* operands, size_t operand_bytes, int iters,
                             void* sink, long long* flop, void* stream) {
     using namespace fo;
@@ -148,8 +166,10 @@ extern "C" int fo_mfma_spin(int dtype, int wide, int traffic, const void* operan
     if ((traffic & 2) && (operand_bytes < (4u << 20) || operand_bytes > 0xffffffffull))
         return fail(FO_ERR_ARG, "fo_mfma_spin: copies need 4 MiB..4 GiB of operands, got %zu bytes", operand_bytes);
     if (iters < 1 || iters > (1 << 20)) return fail(FO_ERR_ARG, "fo_mfma_spin: iters=%d outside 1..2^20", iters);
-    int cus = 0;
-    if (int rc = fo_device_info(&cus, nullptr, nullptr)) return rc;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return fail(FO_ERR_HIP, "fo_mfma_spin: cannot read the CU count of the current device");
     const unsigned n16 = (unsigned)(operand_bytes / 16);
     // the copies walk a power-of-two window of at most half the buffer (and at most 64 MiB)
     unsigned window = 1u << 21;
@@ -168,7 +188,8 @@ extern "C" int fo_mfma_spin(int dtype, int wide, int traffic, const void* operan
     }
     hipLaunchKernelGGL(kern, dim3(cus), dim3(256), 0, (hipStream_t)stream, (const uint4*)operands, n16, iters, window,
                        (float*)sink);
-    FO_HIP(hipGetLastError());
+    if (hipError_t e = hipGetLastError(); e != hipSuccess)
+        return fail(FO_ERR_HIP, "fo_mfma_spin: launch failed: %s", hipGetErrorString(e));
     // one workgroup per CU, 4 wavefronts each, 128 MFMAs of 2*16*16*32 flop (or 64 of 2*32*32*16) per iteration
     if (flop) *flop = (long long)cus * 4 * iters * kSpinMfmas * (2ll * 16 * 16 * 32);
     return FO_OK;

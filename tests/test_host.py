@@ -18,8 +18,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 # ---- C ABI ----------------------------------------------------------------
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "flashoverlap_hip.h")).read()
+def _declared_symbols(header="flashoverlap_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(fo_[a-z0-9_]+)\s*\(", text)))
 
@@ -30,6 +30,17 @@ def test_library_exports_every_declared_symbol(fo_lib):
     for n in names:
         assert hasattr(fo_lib, n), f"{n} is declared in the header but not exported"
     assert sorted(capi.SIGNATURES) == names, "capi.SIGNATURES and the header disagree"
+
+
+def test_probe_library_is_separate_from_the_product(fo_lib):
+    """The measurement probes are a library of their own: declared in their own header, exported
+    by libfo_bench.so, and neither declared nor exported by the product library."""
+    names = _declared_symbols("flashoverlap_bench.h")
+    assert names == sorted(capi.BENCH_SIGNATURES) and "fo_mfma_spin" in names
+    bench = capi.bench_lib()
+    for n in names:
+        assert hasattr(bench, n), f"{n} is declared in flashoverlap_bench.h but not exported"
+        assert n not in capi.SIGNATURES and not hasattr(fo_lib, n), f"{n} leaked into the product library"
 
 
 def test_algo_table_matches_reference_instances(fo_lib):

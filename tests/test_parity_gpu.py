@@ -196,11 +196,13 @@ def test_time_next_launch_gives_the_kernel_duration(L, dev):
 @pytest.mark.parametrize("wide,traffic", [(0, 0), (1, 0), (0, 1), (0, 2), (0, 3)])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wide, traffic):
-    """The MFMA-only loop used as the power-limit yardstick, bare and with a GEMM tile's fragment
+    """(The probe lives in libfo_bench.so, outside the product library; the events are the product's.)
+    The MFMA-only loop used as the power-limit yardstick, bare and with a GEMM tile's fragment
     reads and copies beside it: reads its operands inside the buffer it is given (an odd number
     of 16-byte chunks where it makes no copies, 4 MiB + 16 bytes where it does), reports 128 MFMAs
     x 16384 flop (or 64 x 32768) x 4 wavefronts x CUs per round, writes nothing outside its own
     LDS, and is not faster than the chip."""
+    LB = capi.bench_lib()
     cu = C.c_int()
     capi.check(L.fo_device_info(C.byref(cu), None, None))
     nelem = (4 << 20) // 2 + 8 if traffic & 2 else 7 * 8
@@ -213,9 +215,9 @@ def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wi
     capi.check(L.fo_event_create(C.byref(e0)))
     capi.check(L.fo_event_create(C.byref(e1)))
     args = (capi.dtype_code(dt), wide, traffic, buf.data_ptr(), nelem * 2, iters, guard[32:].data_ptr(), C.byref(flop), None)
-    capi.check(L.fo_mfma_spin(*args))
+    capi.bench_check(LB.fo_mfma_spin(*args))
     capi.check(L.fo_event_record(e0, None))
-    capi.check(L.fo_mfma_spin(*args))
+    capi.bench_check(LB.fo_mfma_spin(*args))
     capi.check(L.fo_event_record(e1, None))
     torch.cuda.synchronize()
     ms = C.c_float()
@@ -226,13 +228,13 @@ def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wi
     rate = flop.value / (ms.value * 1e-3)
     _say("  MFMA loop, wide %d traffic %d: %.0f TFLOP/s" % (wide, traffic, rate / 1e12))
     assert 0.3e15 < rate < 2.6e15
-    assert L.fo_mfma_spin(7, *args[1:]) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], wide, 4, *args[3:]) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], 1, 1, *args[3:]) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], 0, 2, buf.data_ptr(), 1 << 20, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], wide, 0, None, 16, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], wide, 0, buf.data_ptr(), 8, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
-    assert L.fo_mfma_spin(args[0], wide, 0, buf.data_ptr(), 112, 0, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert LB.fo_mfma_spin(7, *args[1:]) == capi.FO_ERR_ARG
+    assert LB.fo_mfma_spin(args[0], wide, 4, *args[3:]) == capi.FO_ERR_ARG
+    assert LB.fo_mfma_spin(args[0], 1, 1, *args[3:]) == capi.FO_ERR_ARG
+    assert LB.fo_mfma_spin(args[0], 0, 2, buf.data_ptr(), 1 << 20, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert LB.fo_mfma_spin(args[0], wide, 0, None, 16, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert LB.fo_mfma_spin(args[0], wide, 0, buf.data_ptr(), 8, 1, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
+    assert LB.fo_mfma_spin(args[0], wide, 0, buf.data_ptr(), 112, 0, guard.data_ptr(), None, None) == capi.FO_ERR_ARG
     capi.check(L.fo_event_destroy(e0))
     capi.check(L.fo_event_destroy(e1))
 
