@@ -216,7 +216,7 @@ def main() -> int:
         if not g.per_group:
             capi.check(L.fo_wait_consume(g.cseg_d.data_ptr(), g.G, g.MM.data_ptr(), Cp.data_ptr(),
                                          staging.data_ptr(), BM * BN, ws, 0, ws, (M * N // ws) if ws > 1 else 0,
-                                         None, a.consumer_blocks, comm))
+                                         None, a.consumer_blocks, None, comm))
             capi.check(L.fo_stream_join(comm, main_stream))
             return
         # like OverlapImpl: the groups before the last are copied beside the GEMM; if that is a lot of data,
@@ -234,13 +234,13 @@ def main() -> int:
                 stream = main_stream
             settle = last_on_main and a.last_group != "main"
             if not settle:
-                capi.check(L.fo_wait(n, g.MM.data_ptr() + 4 * gi, stream))
+                capi.check(L.fo_wait(n, g.MM.data_ptr() + 4 * gi, None, stream))
             elems = n * BM * BN
             part = elems // ws
             # one launch per group (ws > 1: slice k of the group goes to rank k's receive buffer)
             capi.check(L.fo_consume_slices(n, g.MM.data_ptr() + 4 * gi if settle else None, Cp.data_ptr() + 2 * acc,
                                            staging.data_ptr() + 2 * (acc // ws), 2 * part, ws, 2 * (M * N // ws),
-                                           2 if gi == g.G - 1 else beside_policy, stream))
+                                           2 if gi == g.G - 1 else beside_policy, None, stream))
             acc += elems
         if a.last_group == "comm" or (a.last_group == "settle_then_join" and g.G > 1):
             capi.check(L.fo_stream_join(comm, main_stream))
@@ -344,6 +344,14 @@ def main() -> int:
     # no waiter runs here: the group counters simply accumulate and are cleared afterwards
     sig_ms, sig_min = time_kernel(lambda i: gemm_signal(grp), it)
     grp.MM.zero_()
+    # the same launches with the signal in its release-ordered form (the atomic itself a release at
+    # agent scope, which writes the L2's dirty lines back first) instead of the default (write-through
+    # tile stores, acknowledged, a barrier, a relaxed atomic)
+    default_release_mode = next((int(kv.partition("=")[2]) for kv in a.tune if kv.startswith("release_mode=")), 1)
+    capi.check(L.fo_tune(b"release_mode", 0))
+    sig_rel_ms, _ = time_kernel(lambda i: gemm_signal(grp), it)
+    capi.check(L.fo_tune(b"release_mode", default_release_mode))
+    grp.MM.zero_()
     pl_ms, pl_min = time_kernel(lambda i: gemm_plain(), it)
     rms_rot_ms, _ = time_kernel(lambda i: norm(i % npairs), it)      # rotation larger than the memory-side cache
     rms_same_ms, rms_min = time_kernel(lambda i: norm(0), it)         # one pair over and over: served by that cache
@@ -403,6 +411,7 @@ def main() -> int:
     del A0, B0
 
     flops = 2.0 * M * N * K
+    traffic_algorithmic = 2 * (M * K + N * K + M * N)   # A and B read once, C written once
     rms_bytes = 2.0 * (M * N * 2) + N * 2
     cons_bytes = 2.0 * (M * N * 2)
     sig_tf = flops / sig_ms / 1e9
@@ -439,9 +448,10 @@ def main() -> int:
 
     reading = ("tiles" if w == w_tiles else "waves" if w == w_waves else "custom") if a.workload in WAVE_READING else "waves"
     line = {
-        "metric": "signaling-GEMM TFLOP/s", "value": round(flops / step_ms / 1e9, 2), "unit": "TFLOP/s",
+        "metric": "signaling-GEMM path step TFLOP/s", "value": round(flops / step_ms / 1e9, 2), "unit": "TFLOP/s",
         "value_is": "2*M*N*K / whole step time (signalling GEMM || consumer, then reorder+RMSNorm); "
-                    "the GEMM kernel's own rate is roofline.achieved",
+                    "the signalling GEMM kernel's own rate is gemm_kernel_tflops = roofline.achieved",
+        "gemm_kernel_tflops": round(flops / step_gemm_ms / 1e9, 2),
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(step_ms, 5),
         "ms_per_step_with_kernel_events": round(step_probed_ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dts, "data": "synthetic",
@@ -456,8 +466,11 @@ def main() -> int:
         "roofline": {"bound": "mfma", "kernel": "gemm_kernel (signalling), inside the same steps run again with an event pair on its dispatch",
                      "achieved": round(flops / step_gemm_ms / 1e9, 2), "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / step_gemm_ms / 1e9 / PEAK_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload), "avg_us": round(step_gemm_ms * 1e3, 2),
-                     "launches": a.steps},
+                     "avg_us": round(step_gemm_ms * 1e3, 2), "launches": a.steps,
+                     # HBM-side bytes per launch from the tracked counter summary of this workload
+                     # (profiles/); the key is left out for a workload that has none
+                     **({"traffic": MEASURED_TRAFFIC_BYTES[a.workload], "traffic_algorithmic": traffic_algorithmic}
+                        if a.workload in MEASURED_TRAFFIC_BYTES else {})},
         "gemm_signal_serial_step": {"achieved": round(flops / serial_gemm_ms / 1e9, 2), "unit": "TFLOP/s",
                                     "avg_us": round(serial_gemm_ms * 1e3, 2)},
         # the same kernel launched back to back on its own (A and B stay in the 256 MB memory-side cache)
@@ -472,12 +485,20 @@ def main() -> int:
                                      "avg_us": round(z_ms * 1e3, 2),
                                      "note": "same kernel and shape, A = B = 0: not power-limited"},
         "mfma_only_loop": mfma_loop,
+        # both back to back against the plain twin of the same run; "release" is the release-ordered atomic
         "signal_overhead_pct": round((sig_ms / pl_ms - 1.0) * 100.0, 2),
+        "signal_overhead_pct_release": round((sig_rel_ms / pl_ms - 1.0) * 100.0, 2),
+        "signal_form": {"default": "write-through tile stores, acknowledged (vmcnt 0), workgroup barrier, relaxed agent-scope atomic",
+                        "release": "release-ordered agent-scope atomic (L2 write-back first), fo_tune release_mode=0",
+                        "gemm_signal_release_isolated_us": round(sig_rel_ms * 1e3, 2)},
         # headline: back to back over a rotation of buffer pairs that exceeds the memory-side cache
         "reorder_rmsnorm": {"bound": "hbm", "peak": PEAK_HBM_GBPS, "unit": "GB/s", "bytes": rms_bytes,
                             **hbm(rms_rot_ms), "buffer_pairs": npairs,
                             "in_step": hbm(step_norm_ms),
-                            "same_pair_back_to_back": {**hbm(rms_same_ms), "min_single_launch_us": round(rms_min * 1e3, 2)}},
+                            "same_pair_back_to_back": {**hbm(rms_same_ms), "min_single_launch_us": round(rms_min * 1e3, 2)},
+                            # the yardstick of the same run: a plain copy kernel moving the same bytes over the same rotation
+                            "copy_kernel_same_run": {"achieved": round(cons_bytes / cons_ms / 1e6, 1),
+                                                     "frac": round(cons_bytes / cons_ms / 1e6 / PEAK_HBM_GBPS, 4)}},
         "consume_copy": {"achieved": round(cons_bytes / cons_ms / 1e6, 1), "unit": "GB/s",
                          "avg_us": round(cons_ms * 1e3, 2)},
         "other_reading": other,

@@ -31,13 +31,13 @@ SIGNATURES = {
     "fo_build_group_table": (_i, [_vp, _i, _i, _vp, _vp]),
     "fo_raster_hint": (_i, [_i, _i, _i, _ip]),
     "fo_tune": (_i, [C.c_char_p, _i]),
-    "fo_wait": (_i, [_i, _vp, _vp]),
-    "fo_wait_consume": (_i, [_vp, _i, _vp, _vp, _vp, _ll, _i, _i, _i, _ll, _vp, _i, _vp]),
+    "fo_wait": (_i, [_i, _vp, _vp, _vp]),
+    "fo_wait_consume": (_i, [_vp, _i, _vp, _vp, _vp, _ll, _i, _i, _i, _ll, _vp, _i, _vp, _vp]),
     "fo_set_wait_timeout_ms": (_i, [_i]),
     "fo_wait_timeouts": (_i, [_ip, _i]),
     "fo_consume": (_i, [_vp, _vp, _sz, _vp]),
-    "fo_settle_consume": (_i, [_i, _vp, _vp, _vp, _sz, _vp]),
-    "fo_consume_slices": (_i, [_i, _vp, _vp, _vp, _sz, _i, _sz, _i, _vp]),
+    "fo_settle_consume": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp]),
+    "fo_consume_slices": (_i, [_i, _vp, _vp, _vp, _sz, _i, _sz, _i, _vp, _vp]),
     "fo_reorder_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "fo_reorder_rmsnorm_batched": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _f, _vp]),
     "fo_rmsnorm": (_i, [_i, _vp, _vp, _vp, _i, _i, _f, _vp]),

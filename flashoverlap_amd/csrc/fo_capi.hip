@@ -99,13 +99,15 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host) { return raster_hint(
 
 int fo_tune(const char* key, int value) { return tune(key, value); }
 
-int fo_wait(int that, int* addr, void* stream) { return launch_wait(that, addr, (hipStream_t)stream); }
+int fo_wait(int that, int* addr, int* expired, void* stream) {
+    return launch_wait(that, addr, expired, (hipStream_t)stream);
+}
 
 int fo_wait_consume(const int* cseg_dev, int G, int* MM, const void* src, void* dst, long long tile_elems,
                     int nslices, int slice_first, int slice_count, long long slice_stride, int* order_log,
-                    int nblocks, void* stream) {
+                    int nblocks, int* expired, void* stream) {
     return launch_wait_consume(cseg_dev, G, MM, src, dst, tile_elems, nslices, slice_first, slice_count,
-                               slice_stride, order_log, nblocks, (hipStream_t)stream);
+                               slice_stride, order_log, nblocks, expired, (hipStream_t)stream);
 }
 
 int fo_set_wait_timeout_ms(int ms) { return set_wait_timeout_ms(ms); }
@@ -116,15 +118,15 @@ int fo_consume(const void* src, void* dst, size_t bytes, void* stream) {
     return launch_consume(src, dst, bytes, (hipStream_t)stream);
 }
 
-int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t bytes, void* stream) {
+int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t bytes, int* expired, void* stream) {
     if (!addr) return fail(FO_ERR_ARG, "fo_settle_consume: null counter address");
-    return launch_consume(src, dst, bytes, (hipStream_t)stream, that, addr);
+    return launch_consume(src, dst, bytes, (hipStream_t)stream, that, addr, 1, 0, FO_COPY_AUTO, expired);
 }
 
 int fo_consume_slices(int that, int* addr, const void* src, void* dst, size_t slice_bytes, int nslices,
-                      size_t dst_stride_bytes, int store_policy, void* stream) {
+                      size_t dst_stride_bytes, int store_policy, int* expired, void* stream) {
     return launch_consume(src, dst, slice_bytes, (hipStream_t)stream, that, addr, nslices, dst_stride_bytes,
-                          store_policy);
+                          store_policy, expired);
 }
 
 int fo_reorder_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int bs, int dim, int BM, int BN,

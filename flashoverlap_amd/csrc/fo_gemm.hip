@@ -64,6 +64,7 @@
 #include <type_traits>
 
 #include "fo_internal.h"
+#include "fo_knobs.h"
 #include "fo_raster.h"
 
 namespace fo {
@@ -121,11 +122,6 @@ constexpr int kBK = 64;             // k-elements per LDS buffer
 constexpr int kRowBytes = kBK * 2;  // one panel row in LDS: 128 bytes = 8 chunks of 16
 
 enum { kPlain = 0, kSignal = 1, kScatter = 2 };
-
-// Tuning knobs (fo_tune): how the epilogue stores C and how it signals.
-extern int g_copy_streaming_stores;   // fo_sync.hip
-int g_store_mode = 1;    // 0 = cached stores, 1 = agent-scope write-through stores (sc1)
-int g_release_mode = 1;  // 1 = write-through tile stores, acknowledged, then a relaxed atomic; 0 = release-ordered atomic
 
 struct GemmParams {
     const void* A;
@@ -189,8 +185,11 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 // STORE: 0 cached, 1 write-through tile stores; REL: 0 release atomic, 1 relaxed atomic.
-template <typename T, int MT, int MODE, int STORE, int REL>
+// EDGE (plain GEMM only): M and N are arbitrary; the rows and columns of a macro tile that lie
+// outside the matrix are computed on zeros and not stored.
+template <typename T, int MT, int MODE, int STORE, int REL, bool EDGE = false>
 __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
+    static_assert(!EDGE || MODE == kPlain, "only the plain GEMM takes shapes that are not multiples of the layout tile");
     constexpr int WT = MT / 2;               // wave quadrant edge
     constexpr int NB = WT / 16;              // 16x16 MFMA blocks per quadrant edge
     constexpr int NH = NB / 2;               // rows of blocks per half step
@@ -215,8 +214,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     // tile: the last row or column of macro tiles may be half inside.  Such a
     // workgroup runs the full main loop (the waves of the outer half re-read the
     // panel rows of the inner half, so nothing outside the operands is touched)
-    // and only the quadrants inside are stored and signalled.
-    const int valid_m = min(MT, p.M - mt.m * MT), valid_n = min(MT, p.N - mt.n * MT);   // MT or MT / 2
+    // and only the quadrants inside are stored and signalled.  EDGE: M and N are
+    // arbitrary; the panel rows beyond the matrix are zero-filled by the
+    // hardware (see the copy addressing below) and only the rows and columns
+    // inside the matrix are stored.
+    const int valid_m = min(MT, p.M - mt.m * MT), valid_n = min(MT, p.N - mt.n * MT);
     const bool live = wm * WT < valid_m && wn * WT < valid_n;                          // this wave's quadrant
 
     // ---- where this wavefront's quadrant goes -------------------------------
@@ -284,10 +286,23 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     }
     int vo0 = cp_off0, vo1 = cp_off1;   // the offsets in use: the tail pair for the last panel
     const int range = k_rest ? kOutOfRange : (int)0xffffffffu;
-    const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, range, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, range, 0x00020000);
-    const unsigned baseA = (unsigned)(mt.m * MT + ((wave * (LOADS * 8)) & (valid_m - 1))) * (unsigned)K * 2u;
-    const unsigned baseB = (unsigned)(mt.n * MT + ((wave * (LOADS * 8)) & (valid_n - 1))) * (unsigned)K * 2u;
+    // EDGE: the hardware checks only the per-lane part of an offset against the descriptor's range.
+    // So the descriptor of an operand starts at the macro tile's first row and ends with the operand,
+    // the row inside the tile goes into the per-lane part (one addition per copy) and only the k
+    // position stays scalar: a lane whose row lies beyond the matrix is then out of range, fetches
+    // nothing and gets zeros, whatever M and N are.
+    const __amdgpu_buffer_rsrc_t rsrcA =
+        EDGE ? __builtin_amdgcn_make_buffer_rsrc((char*)p.A + (size_t)mt.m * MT * K * 2, 0,
+                                                 (int)((unsigned)(p.M - mt.m * MT) * (unsigned)K * 2u), 0x00020000)
+             : __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, range, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcB =
+        EDGE ? __builtin_amdgcn_make_buffer_rsrc((char*)p.B + (size_t)mt.n * MT * K * 2, 0,
+                                                 (int)((unsigned)(p.N - mt.n * MT) * (unsigned)K * 2u), 0x00020000)
+             : __builtin_amdgcn_make_buffer_rsrc((void*)p.B, 0, range, 0x00020000);
+    const unsigned baseA = EDGE ? (unsigned)(wave * (LOADS * 8)) * (unsigned)K * 2u
+                                : (unsigned)(mt.m * MT + ((wave * (LOADS * 8)) & (valid_m - 1))) * (unsigned)K * 2u;
+    const unsigned baseB = EDGE ? (unsigned)(wave * (LOADS * 8)) * (unsigned)K * 2u
+                                : (unsigned)(mt.n * MT + ((wave * (LOADS * 8)) & (valid_n - 1))) * (unsigned)K * 2u;
     const unsigned slab_bytes = 8u * (unsigned)K * 2u;    // bytes between consecutive slabs
     const int lds_cp = wave * (LOADS * 1024);             // this wave's first slab in a panel
 
@@ -302,12 +317,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int j = H * (LOADS / 2); j < (H + 1) * (LOADS / 2); ++j) {
             const int voff = (j & 1) ? vo1 : vo0;   // LOADS*8 is a multiple of 16: slab parity = j parity
+            const unsigned rows = (ISB ? baseB : baseA) + j * slab_bytes;   // the slab's first row, in bytes
             if constexpr (ISB)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, voff,
-                                                         (int)(baseB + j * slab_bytes + koff), 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, EDGE ? (int)((unsigned)voff + rows) : voff,
+                                                         (int)(EDGE ? koff : rows + koff), 0, 0);
             else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(dst + j * 1024), 16, voff,
-                                                         (int)(baseA + j * slab_bytes + koff), 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(dst + j * 1024), 16, EDGE ? (int)((unsigned)voff + rows) : voff,
+                                                         (int)(EDGE ? koff : rows + koff), 0, 0);
         }
     };
     std::false_type unit_a;
@@ -343,12 +359,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
         unsigned char* dst = smem + slot + lds_cp;
         const unsigned koff = (unsigned)kt * (kBK * 2);
         const int voff = (j & 1) ? vo1 : vo0;
+        const unsigned rows = (ISB ? baseB : baseA) + j * slab_bytes;
         if constexpr (ISB)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, voff,
-                                                     (int)(baseB + j * slab_bytes + koff), 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_void*)(dst + j * 1024), 16, EDGE ? (int)((unsigned)voff + rows) : voff,
+                                                     (int)(EDGE ? koff : rows + koff), 0, 0);
         else
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(dst + j * 1024), 16, voff,
-                                                     (int)(baseA + j * slab_bytes + koff), 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_void*)(dst + j * 1024), 16, EDGE ? (int)((unsigned)voff + rows) : voff,
+                                                     (int)(EDGE ? koff : rows + koff), 0, 0);
     };
     // One fragment read.
     auto read_a = [&](int slot_a, int h, int i) { fa[h][i] = *(const frag*)(smem + slot_a + ko[h] + a_lane + i * BLK); };
@@ -539,6 +556,17 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
             }
             const size_t off = (size_t)row * ld + col0 + cc * 8;
             if (!live) continue;   // a quadrant outside the matrix goes through the motions and stores nothing
+            if constexpr (EDGE) {
+                const int gcol = col0 + cc * 8;
+                if (row >= p.M || gcol >= p.N) continue;
+                if (p.N & 7) {     // rows of D are not 16-byte aligned: element by element
+                    const T* e = (const T*)&v;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        if (gcol + k < p.N) D[off + k] = e[k];
+                    continue;
+                }
+            }
             if constexpr (STORE == 1)
                 __builtin_amdgcn_raw_buffer_store_b128(v, drsrc, (int)(off * 2), 0, 16);  // sc1: write-through
             else
@@ -585,11 +613,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(const GemmParams p) {
     }
 }
 
-template <typename T, int MT, int MODE, int STORE, int REL>
-static int launch_one(const GemmParams& p, hipStream_t stream) {
+template <typename T, int MT, int MODE, int STORE, int REL, bool EDGE = false>
+static int launch_one(const GemmParams& p, const LaunchTimer& timer, hipStream_t stream) {
     constexpr int smem_bytes = 5 * MT * kRowBytes;   // five panel slots: 160 KiB at MT = 256
     static_assert(2 * 4 * 32 * (MT + 16) <= smem_bytes, "epilogue strips must fit in the panel slots");
-    auto kern = gemm_kernel<T, MT, MODE, STORE, REL>;
+    auto kern = gemm_kernel<T, MT, MODE, STORE, REL, EDGE>;
     // The attribute belongs to the function on one device: set it once per device.
     static std::atomic<unsigned long long> configured{0};
     int dev = 0;
@@ -599,10 +627,8 @@ static int launch_one(const GemmParams& p, hipStream_t stream) {
         FO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes));
         configured.fetch_or(bit, std::memory_order_release);
     }
-    if (t_launch_timer.start) {
-        const LaunchTimer t = t_launch_timer;
-        t_launch_timer = LaunchTimer{};
-        hipExtLaunchKernelGGL(kern, dim3(p.GM * p.GN), dim3(256), smem_bytes, stream, t.start, t.stop, 0, p);
+    if (timer.start) {
+        hipExtLaunchKernelGGL(kern, dim3(p.GM * p.GN), dim3(256), smem_bytes, stream, timer.start, timer.stop, 0, p);
     } else {
         hipLaunchKernelGGL(kern, dim3(p.GM * p.GN), dim3(256), smem_bytes, stream, p);
     }
@@ -611,24 +637,29 @@ static int launch_one(const GemmParams& p, hipStream_t stream) {
 }
 
 template <typename T, int MT>
-static int launch_mt(int mode, const GemmParams& p, hipStream_t stream) {
-    const int store = mode == kPlain ? (g_store_mode ? 1 : 0) : (g_store_mode || g_release_mode ? 1 : 0);
-    const int rel = (mode != kPlain && g_release_mode) ? 1 : 0;
+static int launch_mt(int mode, bool edge, const GemmParams& p, const LaunchTimer& timer, hipStream_t stream) {
+    // fo_tune knobs (how the epilogue stores C and how it signals), each read once per launch
+    const int store_mode = knob(knobs().store_mode), release_mode = knob(knobs().release_mode);
+    const int store = mode == kPlain ? (store_mode ? 1 : 0) : (store_mode || release_mode ? 1 : 0);
+    const int rel = (mode != kPlain && release_mode) ? 1 : 0;
+    if (mode == kPlain && edge)
+        return store ? launch_one<T, MT, kPlain, 1, 0, true>(p, timer, stream) : launch_one<T, MT, kPlain, 0, 0, true>(p, timer, stream);
     if (mode == kPlain)
-        return store ? launch_one<T, MT, kPlain, 1, 0>(p, stream) : launch_one<T, MT, kPlain, 0, 0>(p, stream);
+        return store ? launch_one<T, MT, kPlain, 1, 0>(p, timer, stream) : launch_one<T, MT, kPlain, 0, 0>(p, timer, stream);
     if (mode == kSignal) {
-        if (rel) return launch_one<T, MT, kSignal, 1, 1>(p, stream);
-        return store ? launch_one<T, MT, kSignal, 1, 0>(p, stream) : launch_one<T, MT, kSignal, 0, 0>(p, stream);
+        if (rel) return launch_one<T, MT, kSignal, 1, 1>(p, timer, stream);
+        return store ? launch_one<T, MT, kSignal, 1, 0>(p, timer, stream) : launch_one<T, MT, kSignal, 0, 0>(p, timer, stream);
     }
-    if (rel) return launch_one<T, MT, kScatter, 1, 1>(p, stream);
-    return store ? launch_one<T, MT, kScatter, 1, 0>(p, stream) : launch_one<T, MT, kScatter, 0, 0>(p, stream);
+    if (rel) return launch_one<T, MT, kScatter, 1, 1>(p, timer, stream);
+    return store ? launch_one<T, MT, kScatter, 1, 0>(p, timer, stream) : launch_one<T, MT, kScatter, 0, 0>(p, timer, stream);
 }
 
-int choose_macro_tile(int BM, int BN, int M, int N) {
-    if (M % BM || N % BN) return 0;
+int choose_macro_tile(int BM, int BN, int M, int N, bool any_shape) {
+    if (!any_shape && (M % BM || N % BN)) return 0;
     // Every layout tile (128 or 256 on a side) divides the 256x256 macro tile; a matrix edge
-    // that is an odd multiple of 128 is covered by half a macro tile.
-    const bool ok128 = BM == 128 && BN == 128;
+    // that is an odd multiple of 128 is covered by half a macro tile.  The plain GEMM has no
+    // layout to respect: any M and N, either macro tile.
+    const bool ok128 = any_shape || (BM == 128 && BN == 128);
     if (ok128) {
         // Small problems: prefer the tile that puts work on more CUs.
         const int wg256 = ((M + 255) / 256) * ((N + 255) / 256);
@@ -640,6 +671,17 @@ int choose_macro_tile(int BM, int BN, int M, int N) {
 int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg, int G,
                 const int* gtable, const void* A, const void* B, void* D, int* MM, const int* RA,
                 const int* RE, int monitor, hipStream_t stream) {
+    // An event pair armed by fo_time_next_launch belongs to this call whether or not it gets as far
+    // as a launch: taken here, ahead of the validation, so that a rejected call cannot leave it
+    // behind for some later, unrelated launch.
+    const LaunchTimer timer = t_launch_timer;
+    t_launch_timer = LaunchTimer{};
+    if (timer.start) {   // a dispatch that carries events cannot be recorded into a graph
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        FO_HIP(hipStreamIsCapturing(stream, &status));
+        if (status != hipStreamCaptureStatusNone)
+            return fail(FO_ERR_ARG, "fo_gemm: the event pair of fo_time_next_launch cannot be attached while the stream is being captured");
+    }
     int BM, BN, BK;
     if (algo_tile(algo, &BM, &BN, &BK) != FO_OK) return fail(FO_ERR_ARG, "fo_gemm: Algo %d out of range", algo);
     if ((BM != 128 && BM != 256) || (BN != 128 && BN != 256))
@@ -647,17 +689,25 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
     if (dtype != FO_F16 && dtype != FO_BF16) return fail(FO_ERR_ARG, "fo_gemm: dtype %d not fp16/bf16", dtype);
     if (!A || !B || !D) return fail(FO_ERR_ARG, "fo_gemm: null operand");
     if (M <= 0 || N <= 0 || K <= 0) return fail(FO_ERR_SHAPE, "fo_gemm: empty problem %dx%dx%d", M, N, K);
-    if (M % BM || N % BN) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d not multiples of the %dx%d tile", M, N, BM, BN);
+    // The plain GEMM writes a natural row-major D and takes any M and N; the signalling modes place
+    // whole layout tiles.
+    const bool any_shape = mode == kPlain;
+    if (!any_shape && (M % BM || N % BN))
+        return fail(FO_ERR_SHAPE, "fo_gemm_signal: M=%d N=%d not multiples of the %dx%d tile", M, N, BM, BN);
     if (K % 8) return fail(FO_ERR_SHAPE, "fo_gemm: K=%d not a multiple of 8 (operand rows must be 16-byte aligned)", K);
     if ((long long)M * N >= (1LL << 31)) return fail(FO_ERR_LIMIT, "fo_gemm: M*N=%lld needs 64-bit tile offsets", (long long)M * N);
-    if ((long long)M * K >= (1LL << 31) || (long long)N * K >= (1LL << 31))
+    // (the rows a macro tile may reach beyond an operand must still have 32-bit byte offsets)
+    if (((long long)M + 256) * K >= (1LL << 31) || ((long long)N + 256) * K >= (1LL << 31))
         return fail(FO_ERR_LIMIT, "fo_gemm: an operand of %lld elements exceeds the 4 GiB a buffer descriptor addresses",
                     (long long)(M > N ? M : N) * K);
     if (K % kBK && ((long long)M * K >= (1LL << 30) || (long long)N * K >= (1LL << 30)))
         return fail(FO_ERR_LIMIT, "fo_gemm: K=%d is not a multiple of %d and an operand exceeds the 2 GiB this case addresses", K, kBK);
     if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)D) & 15) return fail(FO_ERR_ARG, "fo_gemm: operands must be 16-byte aligned");
-    const int macro = choose_macro_tile(BM, BN, M, N);
+    const int macro = choose_macro_tile(BM, BN, M, N, any_shape);
     if (!macro) return fail(FO_ERR_SHAPE, "fo_gemm: M=%d N=%d not multiples of the %dx%d tile", M, N, BM, BN);
+    // Shapes that are multiples of 128 keep the kernel without row and column predicates (an odd
+    // multiple of 128 is half a macro tile, which that kernel handles by whole quadrants).
+    const bool edge = any_shape && (M % 128 || N % 128);
 
     GemmParams p{};
     p.A = A; p.B = B; p.D = D;
@@ -677,8 +727,9 @@ int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, co
         if (mode == kScatter && !RE) return fail(FO_ERR_ARG, "fo_gemm_scatter: null RE");
     }
     if (dtype == FO_F16)
-        return macro == 256 ? launch_mt<_Float16, 256>(mode, p, stream) : launch_mt<_Float16, 128>(mode, p, stream);
-    return macro == 256 ? launch_mt<__bf16, 256>(mode, p, stream) : launch_mt<__bf16, 128>(mode, p, stream);
+        return macro == 256 ? launch_mt<_Float16, 256>(mode, edge, p, timer, stream)
+                            : launch_mt<_Float16, 128>(mode, edge, p, timer, stream);
+    return macro == 256 ? launch_mt<__bf16, 256>(mode, edge, p, timer, stream) : launch_mt<__bf16, 128>(mode, edge, p, timer, stream);
 }
 
 int raster_hint(int algo, int M, int N, int* hint) {
@@ -686,7 +737,7 @@ int raster_hint(int algo, int M, int N, int* hint) {
     if (algo_tile(algo, &BM, &BN, &BK) != FO_OK) return fail(FO_ERR_ARG, "fo_raster_hint: Algo %d out of range", algo);
     if (!hint) return fail(FO_ERR_ARG, "fo_raster_hint: null hint");
     if (M <= 0 || N <= 0 || M % BM || N % BN) return fail(FO_ERR_SHAPE, "fo_raster_hint: M=%d N=%d vs tile %dx%d", M, N, BM, BN);
-    const int macro = choose_macro_tile(BM, BN, M, N);
+    const int macro = choose_macro_tile(BM, BN, M, N, false);
     if (!macro) return fail(FO_ERR_SHAPE, "fo_raster_hint: M=%d N=%d unsupported for tile %dx%d", M, N, BM, BN);
     const int GM = (M + macro - 1) / macro, GN = (N + macro - 1) / macro, TM = M / BM, TN = N / BN;
     const int tiles_m = macro / BM, tiles_n = macro / BN;
@@ -704,11 +755,7 @@ int raster_hint(int algo, int M, int N, int* hint) {
 
 int tune(const char* key, int value) {
     if (!key) return fail(FO_ERR_ARG, "fo_tune: null key");
-    const std::string_view k(key);
-    if (k == "store_mode") g_store_mode = value ? 1 : 0;
-    else if (k == "release_mode") g_release_mode = value ? 1 : 0;
-    else if (k == "copy_streaming_stores" && value >= 0 && value <= 2) g_copy_streaming_stores = value;
-    else return fail(FO_ERR_ARG, "fo_tune: unknown knob '%s'", key);
+    if (!set_knob(key, value)) return fail(FO_ERR_ARG, "fo_tune: unknown knob '%s' or value %d out of its range", key, value);
     return FO_OK;
 }
 

@@ -30,7 +30,7 @@ struct LaunchTimer {
 extern thread_local LaunchTimer t_launch_timer;
 
 // fo_gemm.hip
-int choose_macro_tile(int BM, int BN, int M, int N);
+int choose_macro_tile(int BM, int BN, int M, int N, bool any_shape);
 int launch_gemm(int mode, int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg, int G,
                 const int* gtable, const void* A, const void* B, void* D, int* MM, const int* RA,
                 const int* RE, int monitor, hipStream_t stream);
@@ -43,12 +43,12 @@ int gemm_signal_static(int dtype, int algo, int M, int N, int K, int rLDN, const
 
 // fo_sync.hip
 int launch_group_table(const int* cseg, int G, int T, int* table, hipStream_t stream);
-int launch_wait(int that, int* addr, hipStream_t stream);
+int launch_wait(int that, int* addr, int* expired, hipStream_t stream);
 int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* dst, long long tile_elems,
                         int nslices, int slice_first, int slice_count, long long slice_stride, int* order_log,
-                        int nblocks, hipStream_t stream);
+                        int nblocks, int* expired, hipStream_t stream);
 int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream, int that = 0, int* addr = nullptr,
-                   int nslices = 1, size_t dst_stride_bytes = 0, int policy = FO_COPY_AUTO);
+                   int nslices = 1, size_t dst_stride_bytes = 0, int policy = FO_COPY_AUTO, int* expired = nullptr);
 int set_wait_timeout_ms(int ms);
 int wait_timeouts(int* count, int reset);
 

@@ -2,7 +2,8 @@
 // the whole row held in registers between the sum of squares and the scaling,
 // 128-bit coalesced HBM accesses, a wavefront butterfly for the reduction (no
 // LDS, no barrier); gamma is fetched together with the row so that nothing but
-// arithmetic sits between the last load and the first store.  The reorder
+// arithmetic sits between the last load and the first store.  (Rows of more
+// than 16384 elements take a second kernel: one workgroup per row, two passes.)  The reorder
 // variant gathers the row from the tile-permuted GEMM output: 16 consecutive
 // lanes read one 256-byte row segment of a 128-wide tile, so every access is
 // made of whole cache lines.  In the common case (rldn == 1, power-of-two tile,
@@ -36,6 +37,29 @@ struct Vec8<__bf16> {
 };
 
 constexpr int kRowsPerBlock = 4;  // one wavefront per row; neighbouring rows read neighbouring tile segments
+constexpr int kWideThreads = 256;  // rows too long for one wavefront's registers: one workgroup per row
+
+template <typename V>
+__device__ __forceinline__ V load_row_chunk(const V* p) {
+#ifdef FO_RMS_LOAD_NT
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+// streaming store by default: the result is not read again here, and it must not displace the
+// GEMM operands held in the memory-side cache
+template <typename V>
+__device__ __forceinline__ void store_row_chunk(V v, V* p) {
+#if defined(FO_RMS_STORE_BITS)
+    typedef unsigned int lab_u32x4 __attribute__((ext_vector_type(4)));
+    asm volatile("global_store_dwordx4 %0, %1, off " FO_RMS_STORE_BITS ::"v"(p), "v"(__builtin_bit_cast(lab_u32x4, v)) : "memory");
+#elif defined(FO_RMS_STORE_PLAIN)
+    *p = v;
+#else
+    __builtin_nontemporal_store(v, p);
+#endif
+}
 
 enum { kNormPlain = 0, kNormGather = 1, kNormGatherFast = 2 };
 
@@ -74,7 +98,7 @@ __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __
             const int s = __shfl(mine, (j >> p.log_bn) & 63, 64);  // all lanes take part in the exchange
             if (c < nchunk) {
                 const size_t src = ((((size_t)s << p.log_bm) + in_row) << p.log_bn) + (j & (p.BN - 1));
-                xv[k] = *(const vec*)(x + src);
+                xv[k] = load_row_chunk((const vec*)(x + src));
             }
         }
     } else if constexpr (MODE == kNormGather) {
@@ -89,7 +113,7 @@ __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __
                 const int j = c << 3;
                 const int s = RA[tile_row + j / p.BN];
                 const size_t src = (size_t)((s / p.rldn) * p.BM + in_row) * ld + (s % p.rldn) * p.BN + j % p.BN;
-                xv[k] = *(const vec*)(x + src);
+                xv[k] = load_row_chunk((const vec*)(x + src));
             }
         }
     } else {
@@ -97,7 +121,7 @@ __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __
 #pragma unroll
         for (int k = 0; k < CH; ++k) {
             const int c = k * 64 + lane;
-            if (c < nchunk) xv[k] = *(const vec*)(xr + (c << 3));
+            if (c < nchunk) xv[k] = load_row_chunk((const vec*)(xr + (c << 3)));
         }
     }
 #pragma unroll
@@ -137,10 +161,67 @@ __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __
                 const T y = (T)((float)xv[k][e] * scale);
                 o[e] = (T)((float)y * (float)gv[k][e]);
             }
-            // streaming store: the result is not read again here, and it must not
-            // displace the GEMM operands held in the memory-side cache
-            __builtin_nontemporal_store(o, (vec*)(orow + (c << 3)));
+            store_row_chunk(o, (vec*)(orow + (c << 3)));
         }
+    }
+}
+
+// Rows longer than a wavefront keeps in registers (dim > 16384): one workgroup per row, two passes.
+// The first pass sums the squares, the four wavefronts' partial sums meet in LDS (added in a fixed
+// order), the second pass reads the row again (it is at most a few hundred KiB and still in the L2)
+// and writes the result.  Same arithmetic per element as above; any dim that is a multiple of 8.
+template <typename T, int MODE>
+__global__ void __launch_bounds__(kWideThreads) rmsnorm_wide_kernel(const T* __restrict__ x0, const T* __restrict__ gamma,
+                                                                  T* __restrict__ out0, const int* __restrict__ RA,
+                                                                  const NormParams p) {
+    static_assert(MODE == kNormPlain || MODE == kNormGather, "rows this long have more than 64 tiles");
+    using vec = typename Vec8<T>::type;
+    __shared__ float part[kWideThreads / 64];
+    const int row = blockIdx.x;
+    const T* __restrict__ x = x0 + (size_t)blockIdx.y * p.bs * p.dim;
+    T* __restrict__ orow = out0 + (size_t)blockIdx.y * p.bs * p.dim + (size_t)row * p.dim;
+    const int dim = p.dim, nchunk = dim >> 3;
+    [[maybe_unused]] const int ldn = MODE == kNormGather ? dim / p.BN : 0;
+    [[maybe_unused]] const int tile_row = MODE == kNormGather ? (row / p.BM) * ldn : 0;
+    [[maybe_unused]] const int in_row = MODE == kNormGather ? row % p.BM : 0;
+    auto chunk_at = [&](int c) -> const vec* {
+        const int j = c << 3;
+        if constexpr (MODE == kNormGather) {
+            const int s = RA[tile_row + j / p.BN];
+            return (const vec*)(x + (size_t)((s / p.rldn) * p.BM + in_row) * (p.rldn * p.BN) + (s % p.rldn) * p.BN + j % p.BN);
+        } else {
+            return (const vec*)(x + (size_t)row * dim + j);
+        }
+    };
+    float ss = 0.f;
+#pragma unroll 4
+    for (int c = threadIdx.x; c < nchunk; c += kWideThreads) {
+        const vec v = *chunk_at(c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float f = (float)v[e];
+            ss += f * f;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = part[0];
+#pragma unroll
+    for (int w = 1; w < kWideThreads / 64; ++w) total += part[w];
+    const float scale = rsqrtf(total / (float)dim + p.eps);
+#pragma unroll 4
+    for (int c = threadIdx.x; c < nchunk; c += kWideThreads) {
+        const vec v = *chunk_at(c);
+        const vec g = *(const vec*)(gamma + (c << 3));
+        vec o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const T y = (T)((float)v[e] * scale);
+            o[e] = (T)((float)y * (float)g[e]);
+        }
+        store_row_chunk(o, (vec*)(orow + (c << 3)));
     }
 }
 
@@ -152,12 +233,28 @@ static int log2_exact(int v) {
 }
 
 template <typename T, int MODE>
+static int launch_wide(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p, int nbatch,
+                       const LaunchTimer& timer, hipStream_t stream) {
+    const dim3 grid(p.bs, nbatch), block(kWideThreads);
+    if (timer.start)
+        hipExtLaunchKernelGGL((rmsnorm_wide_kernel<T, MODE>), grid, block, 0, stream, timer.start, timer.stop, 0,
+                              (const T*)x, (const T*)gamma, (T*)out, RA, p);
+    else
+        hipLaunchKernelGGL((rmsnorm_wide_kernel<T, MODE>), grid, block, 0, stream, (const T*)x, (const T*)gamma, (T*)out,
+                           RA, p);
+    FO_HIP(hipGetLastError());
+    return FO_OK;
+}
+
+template <typename T, int MODE>
 static int launch_t(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p, int nbatch,
-                    hipStream_t stream) {
+                    const LaunchTimer& timer, hipStream_t stream) {
     const int ch = (p.dim / 8 + 63) / 64;
+    if (ch > 32) {   // beyond what a wavefront keeps in registers
+        if constexpr (MODE == kNormGatherFast) return fail(FO_ERR_SHAPE, "fo_reorder_rmsnorm: dim=%d", p.dim);   // not selected for such rows
+        else return launch_wide<T, MODE>(x, gamma, out, RA, p, nbatch, timer, stream);
+    }
     const dim3 grid((p.bs + kRowsPerBlock - 1) / kRowsPerBlock, nbatch), block(64 * kRowsPerBlock);
-    const LaunchTimer timer = t_launch_timer;
-    t_launch_timer = LaunchTimer{};
 #define FO_RMS_CASE(CH)                                                                                           \
     do {                                                                                                          \
         if (timer.start)                                                                                          \
@@ -180,23 +277,26 @@ static int launch_t(const void* x, const void* gamma, void* out, const int* RA, 
 
 template <typename T>
 static int launch_dtype(const void* x, const void* gamma, void* out, const int* RA, const NormParams& p, int nbatch,
-                        hipStream_t stream) {
-    if (!RA) return launch_t<T, kNormPlain>(x, gamma, out, RA, p, nbatch, stream);
-    if (p.log_bm >= 0) return launch_t<T, kNormGatherFast>(x, gamma, out, RA, p, nbatch, stream);
-    return launch_t<T, kNormGather>(x, gamma, out, RA, p, nbatch, stream);
+                        const LaunchTimer& timer, hipStream_t stream) {
+    if (!RA) return launch_t<T, kNormPlain>(x, gamma, out, RA, p, nbatch, timer, stream);
+    if (p.log_bm >= 0) return launch_t<T, kNormGatherFast>(x, gamma, out, RA, p, nbatch, timer, stream);
+    return launch_t<T, kNormGather>(x, gamma, out, RA, p, nbatch, timer, stream);
 }
 
 int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int nbatch, int bs, int dim, int BM,
                    int BN, int rldn, const int* RA, float eps, hipStream_t stream) {
     const bool reorder = RA != nullptr;
     const char* who = reorder ? "fo_reorder_rmsnorm" : "fo_rmsnorm";
+    // an event pair armed by fo_time_next_launch is this call's, whether or not it gets as far as a launch
+    const LaunchTimer timer = t_launch_timer;
+    t_launch_timer = LaunchTimer{};
     if (dtype != FO_F16 && dtype != FO_BF16) return fail(FO_ERR_ARG, "%s: dtype %d not fp16/bf16", who, dtype);
     if (bs == 0 || nbatch == 0) return FO_OK;
     if (nbatch < 0 || nbatch > 65535) return fail(FO_ERR_LIMIT, "%s: %d batches outside 0..65535", who, nbatch);
     if (!x || !gamma || !out) return fail(FO_ERR_ARG, "%s: null buffer", who);
     if (bs < 0 || dim <= 0) return fail(FO_ERR_SHAPE, "%s: bs=%d dim=%d", who, bs, dim);
     if (dim % 8) return fail(FO_ERR_SHAPE, "%s: dim=%d not a multiple of 8", who, dim);
-    if (dim > 32 * 512) return fail(FO_ERR_LIMIT, "%s: dim=%d above the 16384 a wavefront keeps in registers", who, dim);
+    if ((long long)bs * dim * nbatch >= (1LL << 40)) return fail(FO_ERR_LIMIT, "%s: %lld elements", who, (long long)bs * dim * nbatch);
     if (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)out) & 15) return fail(FO_ERR_ARG, "%s: buffers must be 16-byte aligned", who);
     NormParams p{bs, dim, BM, BN, rldn, -1, -1, eps};
     if (reorder) {
@@ -204,13 +304,13 @@ int launch_rmsnorm(int dtype, const void* x, const void* gamma, void* out, int n
         if (BN % 8 || dim % BN) return fail(FO_ERR_SHAPE, "%s: BN=%d must be a multiple of 8 that divides dim=%d", who, BN, dim);
         if (bs % BM) return fail(FO_ERR_SHAPE, "%s: bs=%d not a multiple of BM=%d", who, bs, BM);
         if (((long long)(bs / BM) * (dim / BN)) % rldn) return fail(FO_ERR_SHAPE, "%s: rldn=%d must divide the tile count", who, rldn);
-        if (rldn == 1 && dim / BN <= 64 && log2_exact(BM) >= 0 && log2_exact(BN) >= 0) {
+        if (rldn == 1 && dim / BN <= 64 && dim <= 32 * 512 && log2_exact(BM) >= 0 && log2_exact(BN) >= 0) {
             p.log_bm = log2_exact(BM);
             p.log_bn = log2_exact(BN);
         }
     }
-    if (dtype == FO_F16) return launch_dtype<_Float16>(x, gamma, out, RA, p, nbatch, stream);
-    return launch_dtype<__bf16>(x, gamma, out, RA, p, nbatch, stream);
+    if (dtype == FO_F16) return launch_dtype<_Float16>(x, gamma, out, RA, p, nbatch, timer, stream);
+    return launch_dtype<__bf16>(x, gamma, out, RA, p, nbatch, timer, stream);
 }
 
 }  // namespace fo

@@ -45,6 +45,9 @@ static int scratch_for_current_device(int** out) {
 
 int gemm_signal_static(int dtype, int algo, int M, int N, int K, int rLDN, const int* cseg, int G, const void* A,
                        const void* B, void* D, int* MM, const int* RA, int monitor, hipStream_t stream) {
+    // an event pair armed by fo_time_next_launch is this call's, also if the call is rejected below
+    const LaunchTimer timer = t_launch_timer;
+    t_launch_timer = LaunchTimer{};
     int BM, BN, BK;
     if (algo_tile(algo, &BM, &BN, &BK) != FO_OK) return fail(FO_ERR_ARG, "fo_gemm_signal_static: Algo %d out of range", algo);
     if (M <= 0 || N <= 0 || M % BM || N % BN)
@@ -57,6 +60,7 @@ int gemm_signal_static(int dtype, int algo, int M, int N, int K, int rLDN, const
     int* table = nullptr;
     if (int e = scratch_for_current_device(&table)) return e;
     if (int e = launch_group_table(cseg, G, (int)T, table, stream)) return e;
+    t_launch_timer = timer;   // for the GEMM's own dispatch
     return launch_gemm(1, dtype, algo, M, N, K, rLDN, cseg, G, table, A, B, D, MM, RA, nullptr, monitor, stream);
 }
 

@@ -1,9 +1,13 @@
 // Counter side of the overlap protocol: the wait (counting) kernel, the
 // persistent wait+consume kernel, the consumer copy and the slot->group table.
 //
-// The GEMM epilogue bumps MM[g] with a release-ordered agent-scope atomic once
-// a tile of group g is visible device-wide.  The kernels here run on a second
-// stream while the GEMM is still executing.  MI355X has one L2 per XCD and they
+// The GEMM epilogue bumps MM[g] once a tile of group g is visible device-wide:
+// by default its tile stores are agent-scope write-through stores whose
+// acknowledgement every wavefront waits for, then the workgroup meets at a
+// barrier and a relaxed agent-scope atomic moves the counter (the
+// release-ordered atomic is a tuning knob of the GEMM, not what runs by
+// default).  The kernels here run on a second stream while the GEMM is still
+// executing.  MI355X has one L2 per XCD and they
 // are not coherent with each other, so a reader on another XCD must not hit a
 // stale line.  An acquire would do that by invalidating its caches - including
 // the A/B panels that the GEMM workgroups of that XCD are sharing through the
@@ -18,23 +22,28 @@
 #include <atomic>
 
 #include "fo_internal.h"
+#include "fo_knobs.h"
 
 namespace fo {
 
+// Expired waits are counted in the word the caller passes (`expired`, one that it owns: the count
+// of its own calls) or, if it passes none, in this per-device word (fo_wait_timeouts).
 __device__ int g_wait_timeouts = 0;
 
-static int g_timeout_ms = 10000;
-int g_copy_streaming_stores = 2;   // fo_tune "copy_streaming_stores": 0 never, 1 always, 2 chosen per launch
+__device__ __forceinline__ void count_expired(int* expired) { atomicAdd(expired ? expired : &g_wait_timeouts, 1); }
 
 // Bounded poll of *addr until pred(value); returns false on expiry.
 template <typename Pred>
-__device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, Pred pred) {
+__device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, Pred pred, int nap = 0) {
     const long long t0 = wall_clock64();
     for (;;) {
         const int v = __hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (pred(v)) return true;
         if (wall_clock64() - t0 > ticks) return false;
-        __builtin_amdgcn_s_sleep(8);
+        if (nap <= 0) __builtin_amdgcn_s_sleep(8);
+        else if (nap == 1) __builtin_amdgcn_s_sleep(32);
+        else
+            for (int i = 0; i < (nap >= 4 ? 4 : nap >= 3 ? 2 : 1); ++i) __builtin_amdgcn_s_sleep(127);
     }
 }
 
@@ -43,12 +52,12 @@ __device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, P
 // the last tile's signal and the reset, so load-then-store equals the
 // reference's compare-and-swap.  The kernel that follows on the stream sees
 // the group's tiles through the cache invalidation at its own start.
-__global__ void wait_kernel(int that, int* addr, long long ticks) {
+__global__ void wait_kernel(int that, int* addr, long long ticks, int* expired) {
     if (threadIdx.x != 0) return;
     if (bounded_poll(addr, ticks, [that](int v) { return v == that; }))
         __hip_atomic_store(addr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else
-        atomicAdd(&g_wait_timeouts, 1);
+        count_expired(expired);
 }
 
 constexpr int kCopyThreads = 512;  // workgroup size of the per-group copy kernel
@@ -114,19 +123,29 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
 // dst + (k - slice_first)*stride + offset/nslices (the receive layout of a
 // ReduceScatter; nslices = 1 is the plain copy).
 //
-// The kernel uses no LDS and no workgroup barrier, and few registers: the GEMM
-// workgroup that runs on the same CU owns all of its LDS and most of its
-// registers, and these wavefronts have to fit beside it.  Each wavefront finds
+// The kernel uses no LDS and few registers: the GEMM workgroup that runs on the
+// same CU owns all of its LDS and most of its registers, and these wavefronts
+// have to fit beside it.  Each wavefront finds
 // its groups on its own: 64 groups at a time, one per lane, with wavefront
 // scans for the group offsets and the team windows.
-template <bool STREAM>
+//
+// BY_WG: the members are the workgroups instead of the wavefronts (a team then has one workgroup
+// per 128 KiB of the group).  Only the first wavefront of a member polls; the other three wait at
+// a workgroup barrier, which costs the SIMDs they share with the GEMM no issue slots and the
+// memory system a quarter of the polls.  The barrier needs no LDS.  The poller's result cannot
+// be handed to the other wavefronts without LDS, so after an expired wait the workgroup goes
+// on: it copies the incomplete group (as the copy behind an expired wait kernel does) and polls
+// every later group just once.
+template <bool STREAM, bool BY_WG>
 __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
     const int* __restrict__ cseg, int G, int* MM, const uint4* __restrict__ src, uint4* __restrict__ dst,
     long long tile_units, int nslices, int slice_first, int slice_count, long long slice_stride_units,
-    int* order_log, long long ticks) {
+    int* order_log, long long ticks, int* expired, int nap) {
     const int lane = threadIdx.x & 63;
-    const int self = __builtin_amdgcn_readfirstlane((int)blockIdx.x * kWavesPerBlock + (int)(threadIdx.x >> 6));
-    const int members = (int)gridDim.x * kWavesPerBlock;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int self = BY_WG ? (int)blockIdx.x : (int)blockIdx.x * kWavesPerBlock + wave;
+    const int members = BY_WG ? (int)gridDim.x : (int)gridDim.x * kWavesPerBlock;
+    constexpr long long kPerMember = BY_WG ? kUnitsPerMember * kWavesPerBlock : kUnitsPerMember;
     long long lo_base = 0;  // first 16-byte unit of the chunk's first group
     int start_base = 0;     // first member of that group's team
     for (int g0 = 0; g0 < G; g0 += 64) {
@@ -135,7 +154,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
         const long long units = tile_units * count;
         int team = 0;
         if (g < G) {
-            const long long want = (units + kUnitsPerMember - 1) / kUnitsPerMember;
+            const long long want = (units + kPerMember - 1) / kPerMember;
             team = (int)(want < 1 ? 1 : (want > members ? members : want));
         }
         // inclusive scans of units and team sizes over the 64 groups of the chunk
@@ -162,10 +181,10 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
             const int tm = __shfl(team, b, 64), mem = __shfl(me, b, 64), need = __shfl(count, b, 64);
             const long long glo = __shfl(lo, b, 64);
             int ok = 0;
-            if (lane == 0) {
-                ok = bounded_poll(MM + gg, ticks, [need](int v) { return v >= need; }) ? 1 : 0;
+            if (lane == 0 && (!BY_WG || wave == 0)) {
+                ok = bounded_poll(MM + gg, ticks, [need](int v) { return v >= need; }, nap) ? 1 : 0;
                 if (!ok) {
-                    atomicAdd(&g_wait_timeouts, 1);
+                    count_expired(expired);
                 } else {
                     // Every member has seen the full count once it has bumped it; the last one
                     // to do so puts the counter back.  The copies need not be finished for that:
@@ -180,11 +199,20 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
                     }
                 }
             }
-            if (!__shfl(ok, 0, 64)) return;  // the wait expired: this wavefront gives up on the rest
             const long long part = tile_units * need / nslices;
-            for (int k = 0; k < slice_count; ++k)
-                team_copy<true, 64, STREAM>(src + glo + (slice_first + k) * part,
-                                            dst + k * slice_stride_units + glo / nslices, part, mem, tm, lane);
+            if constexpr (BY_WG) {
+                if (wave == 0 && !__shfl(ok, 0, 64)) ticks = -1;   // every later poll looks once and gives up
+                __builtin_amdgcn_s_barrier();                       // the three other wavefronts slept here
+                for (int k = 0; k < slice_count; ++k)
+                    team_copy<true, 64 * kWavesPerBlock, STREAM>(src + glo + (slice_first + k) * part,
+                                                                 dst + k * slice_stride_units + glo / nslices, part, mem,
+                                                                 tm, (int)threadIdx.x);
+            } else {
+                if (!__shfl(ok, 0, 64)) return;  // the wait expired: this wavefront gives up on the rest
+                for (int k = 0; k < slice_count; ++k)
+                    team_copy<true, 64, STREAM>(src + glo + (slice_first + k) * part,
+                                                dst + k * slice_stride_units + glo / nslices, part, mem, tm, lane);
+            }
         }
         lo_base += __shfl(su, 63, 64);
         start_base = (int)(((long long)start_base + __shfl(st, 63, 64)) % members);
@@ -197,7 +225,7 @@ template <bool STREAM>
 __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
                                                                long long units, long long dst_stride_units,
                                                                const unsigned short* src_tail, unsigned short* dst_tail,
-                                                               int tail, int that, int* addr) {
+                                                               int tail, int that, int* addr, int* expired) {
     // Settling a counter whose producer ran earlier on this stream takes no
     // waiting: it holds its final value.  The right value is cleared like
     // wait_kernel does; a wrong one is left and counted like an expired wait.
@@ -205,7 +233,7 @@ __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __re
         if (__hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == that)
             __hip_atomic_store(addr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else
-            atomicAdd(&g_wait_timeouts, 1);
+            count_expired(expired);
     }
     team_copy<false, kCopyThreads, STREAM>(src + blockIdx.y * units, dst + blockIdx.y * dst_stride_units, units,
                                            blockIdx.x, gridDim.x, threadIdx.x);
@@ -270,13 +298,12 @@ static int device_facts(const DeviceFacts** out) {
 static int ticks_for_timeout(long long* ticks) {
     const DeviceFacts* f;
     if (int e = device_facts(&f)) return e;
-    *ticks = (long long)g_timeout_ms * f->wall_khz;
+    *ticks = (long long)knob(knobs().wait_timeout_ms) * f->wall_khz;
     return FO_OK;
 }
 
 int set_wait_timeout_ms(int ms) {
-    if (ms <= 0) return fail(FO_ERR_ARG, "fo_set_wait_timeout_ms: %d ms", ms);
-    g_timeout_ms = ms;
+    if (!set_wait_timeout(ms)) return fail(FO_ERR_ARG, "fo_set_wait_timeout_ms: %d ms", ms);
     return FO_OK;
 }
 
@@ -291,18 +318,18 @@ int wait_timeouts(int* count, int reset) {
     return FO_OK;
 }
 
-int launch_wait(int that, int* addr, hipStream_t stream) {
+int launch_wait(int that, int* addr, int* expired, hipStream_t stream) {
     if (!addr) return fail(FO_ERR_ARG, "fo_wait: null counter address");
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
-    hipLaunchKernelGGL(wait_kernel, dim3(1), dim3(64), 0, stream, that, addr, ticks);
+    hipLaunchKernelGGL(wait_kernel, dim3(1), dim3(64), 0, stream, that, addr, ticks, expired);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }
 
 int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* dst, long long tile_elems,
                         int nslices, int slice_first, int slice_count, long long slice_stride, int* order_log,
-                        int nblocks, hipStream_t stream) {
+                        int nblocks, int* expired, hipStream_t stream) {
     if (!cseg || !MM || !src || !dst) return fail(FO_ERR_ARG, "fo_wait_consume: null argument");
     if (G <= 0 || nslices <= 0 || tile_elems <= 0) return fail(FO_ERR_ARG, "fo_wait_consume: G=%d nslices=%d tile_elems=%lld", G, nslices, tile_elems);
     if (nblocks <= 0) return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d", nblocks);
@@ -319,15 +346,19 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
         return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d outside 1..%d (one workgroup per CU)", nblocks, facts->cus);
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
-    auto kern = g_copy_streaming_stores ? wait_consume_kernel<true> : wait_consume_kernel<false>;   // runs beside the GEMM
+    const bool streaming = knob(knobs().copy_streaming_stores) != 0;   // it runs beside the GEMM
+    const bool by_wg = knob(knobs().consumer_poll) != 0;
+    auto kern = by_wg ? (streaming ? wait_consume_kernel<true, true> : wait_consume_kernel<false, true>)
+                      : (streaming ? wait_consume_kernel<true, false> : wait_consume_kernel<false, false>);
     hipLaunchKernelGGL(kern, dim3(nblocks), dim3(64 * kWavesPerBlock), 0, stream, cseg, G, MM, (const uint4*)src,
-                       (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks);
+                       (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks,
+                       expired, knob(knobs().poll_nap));
     FO_HIP(hipGetLastError());
     return FO_OK;
 }
 
 int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream, int that, int* addr, int nslices,
-                   size_t dst_stride_bytes, int policy) {
+                   size_t dst_stride_bytes, int policy, int* expired) {
     const char* who = nslices > 1 ? "fo_consume_slices" : "fo_consume";
     if (nslices <= 0 || nslices > 65535) return fail(FO_ERR_ARG, "%s: %d slices outside 1..65535", who, nslices);
     if (bytes == 0 && !addr) return FO_OK;
@@ -353,12 +384,12 @@ int launch_consume(const void* src, void* dst, size_t bytes, hipStream_t stream,
     constexpr size_t kStreamFrom = 48u << 20;
     bool stream_stores = policy == FO_COPY_STREAM ||
                          (policy == FO_COPY_AUTO && !addr && bytes * (size_t)nslices >= kStreamFrom);
-    if (g_copy_streaming_stores != 2) stream_stores = g_copy_streaming_stores == 1;   // forced by fo_tune
+    if (const int forced = knob(knobs().copy_streaming_stores); forced != 2) stream_stores = forced == 1;   // fo_tune
     auto kern = stream_stores ? consume_kernel<true> : consume_kernel<false>;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks, (unsigned)nslices), dim3(kCopyThreads), 0, stream, (const uint4*)src,
                        (uint4*)dst, (long long)units, (long long)(dst_stride_bytes / 16),
                        (const unsigned short*)((const char*)src + units * 16),
-                       (unsigned short*)((char*)dst + units * 16), tail, that, addr);
+                       (unsigned short*)((char*)dst + units * 16), tail, that, addr, expired);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }

@@ -69,9 +69,23 @@ void OverlapImpl::SetWaitTimeoutMs(int64_t ms) {
     FO_CALL(fo_set_wait_timeout_ms((int)ms));
 }
 
+// The word this object's waits count their expiries in (one int32 on the device of `like`).
+int* OverlapImpl::expired_word(const at::Tensor& like) {
+    if (!expired_.defined() || expired_.device() != like.device()) {
+        expired_ = at::zeros({1}, like.options().dtype(at::kInt));
+        // once per object: the fill runs on torch's current stream, the waits on another one
+        c10::hip::getCurrentHIPStream().synchronize();
+    }
+    return expired_.data_ptr<int>();
+}
+
 int64_t OverlapImpl::WaitTimeouts(bool reset) {
-    int n = 0;
-    FO_CALL(fo_wait_timeouts(&n, reset ? 1 : 0));
+    if (!expired_.defined()) return 0;   // no overlapped call has run yet
+    c10::DeviceGuard guard(expired_.device());
+    if (comm_stream_) FO_CALL(fo_stream_sync(comm_stream_));
+    if (gemm_ready_) FO_CALL(fo_stream_sync(gemm_stream_));
+    const int64_t n = expired_.item<int>();
+    if (reset && n) expired_.zero_();
     return n;
 }
 
@@ -82,10 +96,10 @@ void OverlapImpl::SetCheckTimeouts(bool on) { check_timeouts_ = on; }
 // wait on them expire too (or pass at once), so they are cleared here.
 void OverlapImpl::raise_on_timeout(at::Tensor& MM, const char* who) {
     if (!check_timeouts_) return;
-    FO_CALL(fo_stream_sync(gemm_stream_));
-    int n = 0;
-    FO_CALL(fo_wait_timeouts(&n, 1));
+    FO_CALL(fo_stream_sync(gemm_stream_));   // the call's join has ordered it behind the second stream
+    const int n = expired_.item<int>();
     if (n == 0) return;
+    expired_.zero_();
     MM.zero_();
     TORCH_CHECK(false, who, ": ", n, " bounded wait(s) expired before their group completed; the consumer's output "
                 "is incomplete and MM has been zeroed (a cSeg that does not match the tiles, or a GEMM slower than the "
@@ -152,6 +166,25 @@ void OverlapImpl::Gemm(at::Tensor A, at::Tensor B, at::Tensor C, int64_t Algo) {
 // second stream, and with the join at the end the call is a closed fork/join pattern of
 // kernels.  Outside a capture the fork is left out, as in the reference: the event it puts in
 // front of the GEMM costs 5-9 us of every call.
+// Ahead of the GEMM launch of an overlapped call: the word its waits count their expiries in
+// exists (creating it waits for the stream once per object, which must not happen between the
+// GEMM and its waiters), and checked mode is not combined with a capture.
+void OverlapImpl::prepare_call(const at::Tensor& MM, const char* who) {
+    refuse_checked_capture(who);
+    expired_word(MM);
+}
+
+// Checked mode ends every call with a wait for the stream, which a capture forbids (it would
+// invalidate the capture and leave the caller with an unrelated error).
+void OverlapImpl::refuse_checked_capture(const char* who) {
+    if (!check_timeouts_) return;
+    int capturing = 0;
+    FO_CALL(fo_stream_is_capturing(gemm_stream_, &capturing));
+    TORCH_CHECK(!capturing, who, ": set_check_timeouts(true) makes the call wait for its own completion, which is not "
+                "allowed while the stream is being captured into a graph; turn it off for captured calls and read "
+                "wait_timeouts() after a replay instead");
+}
+
 void OverlapImpl::fork_comm_stream(int G) {
     const bool persistent = consumer_mode_ == 2 || (consumer_mode_ == 0 && G > 32);
     if (!persistent && G <= 1) return;   // the second stream is not used
@@ -171,10 +204,11 @@ void OverlapImpl::consume_groups(const at::Tensor& C, void* dst, int64_t tile_el
     const int slice_first = slice_stride ? 0 : (int)my_rank_;      // stride 0: only this rank's slice
     const int slice_count = slice_stride ? nslices : 1;
     const bool persistent = consumer_mode_ == 2 || (consumer_mode_ == 0 && G > 32);
+    int* expired = expired_.data_ptr<int>();   // this object's own count of expired waits (prepare_call)
     if (persistent) {
         FO_CALL(fo_wait_consume(cseg_gpu.data_ptr<int>(), G, MM.data_ptr<int>(), C.data_ptr(), dst, tile_elems,
                                 nslices, slice_first, slice_count, slice_stride, nullptr, consumer_blocks(),
-                                comm_stream_));
+                                expired, comm_stream_));
         // The caller's stream continues only after the last group is consumed
         // (src/overlap_impl.cu:267-270).
         FO_CALL(fo_stream_join(comm_stream_, gemm_stream_));
@@ -198,14 +232,14 @@ void OverlapImpl::consume_groups(const at::Tensor& C, void* dst, int64_t tile_el
         const bool last = g == G - 1;
         void* stream = last ? gemm_stream_ : comm_stream_;
         const int64_t comm = tile_elems * cseg[g];
-        if (!last) FO_CALL(fo_wait(cseg[g], MM.data_ptr<int>() + g, stream));
+        if (!last) FO_CALL(fo_wait(cseg[g], MM.data_ptr<int>() + g, expired, stream));
         // One launch per group, like the one collective call per group of the reference: this
         // rank's slice of the group, or all ranks' slices into their receive buffers side by side.
         const int64_t part = comm / nslices;
         FO_CALL(fo_consume_slices(cseg[g], last ? MM.data_ptr<int>() + g : nullptr,
                                   src + (acc + slice_first * part) * esz, (char*)dst + (acc / nslices) * esz,
                                   part * esz, slice_count, slice_stride * esz,
-                                  last ? FO_COPY_CACHED : beside_policy, stream));
+                                  last ? FO_COPY_CACHED : beside_policy, expired, stream));
         acc += comm;
     }
     // The caller's stream continues only after every group is consumed (src/overlap_impl.cu:267-270).
@@ -221,6 +255,7 @@ void OverlapImpl::GemmAllReduceOverlap(at::Tensor A, at::Tensor B, at::Tensor C,
         fo_host::check_signal(s, MM, RA, at::Tensor(), rLDN, cSEG_CPU, cSEG_GPU, (int)Algo, if_monitor, 1,
                               "gemm_allreduce_overlap");
     c10::DeviceGuard guard(A.device());
+    prepare_call(MM, "gemm_allreduce_overlap");
     at::Tensor& staging = staging_like(C);
     const int* table = group_table_for(cSEG_CPU, cSEG_GPU, g.T);
     fork_comm_stream(g.G);
@@ -247,6 +282,7 @@ void OverlapImpl::GemmReduceScatterOverlap(at::Tensor A, at::Tensor B, at::Tenso
                 "gemm_reducescatter_overlap: D must hold M*N/world_size = ", total / my_size_, " or M*N = ", total,
                 " elements, got ", D.numel());
     c10::DeviceGuard guard(A.device());
+    prepare_call(MM, "gemm_reducescatter_overlap");
     const int* table = group_table_for(cSEG_CPU, cSEG_GPU, g.T);
     fork_comm_stream(g.G);
     FO_CALL(fo_gemm_scatter(s.dtype, (int)Algo, s.M, s.N, s.K, (int)rLDN, cSEG_GPU.data_ptr<int>(), g.G, table,

@@ -62,10 +62,13 @@ class OverlapImpl : public torch::CustomClassHolder {
     void SetConsumerBlocks(int64_t blocks);
     // The waits on the group counters are bounded (the reference's spin forever,
     // src/wait.cuh:6-8).  set_wait_timeout_ms sets the bound (process-wide, default
-    // 10 s); wait_timeouts(reset) synchronises the device and returns how many
-    // waits have expired on it; set_check_timeouts(true) makes every overlapped call
+    // 10 s).  Expired waits are counted in a device word that this object owns, so
+    // one object never sees, or is blamed for, another object's expiries:
+    // wait_timeouts(reset) waits for this object's streams and returns how many of
+    // its waits have expired; set_check_timeouts(true) makes every overlapped call
     // wait for its own completion and raise if one of its waits expired (debugging:
-    // it serialises the caller).  After an expiry MM must be zeroed before reuse.
+    // it serialises the caller, and it cannot be combined with graph capture, which
+    // forbids that wait).  After an expiry MM must be zeroed before reuse.
     void SetWaitTimeoutMs(int64_t ms);
     int64_t WaitTimeouts(bool reset);
     void SetCheckTimeouts(bool on);
@@ -81,6 +84,7 @@ class OverlapImpl : public torch::CustomClassHolder {
     bool check_timeouts_ = false;
 
     at::Tensor staging_;
+    at::Tensor expired_;          // one int32 on the device: expired waits of this object's calls
     at::Tensor group_table_;
     std::vector<int> table_key_;  // cSeg contents + T the table was built for
 
@@ -92,6 +96,9 @@ class OverlapImpl : public torch::CustomClassHolder {
     void consume_groups(const at::Tensor& C, void* dst, int64_t tile_elems, const at::Tensor& cseg_cpu,
                         const at::Tensor& cseg_gpu, at::Tensor& MM, int nslices, int64_t slice_stride);
     void bulk_consume(const void* src, void* dst, size_t bytes);
+    int* expired_word(const at::Tensor& like);
+    void refuse_checked_capture(const char* who);
+    void prepare_call(const at::Tensor& MM, const char* who);
     void raise_on_timeout(at::Tensor& MM, const char* who);
     int consumer_blocks();
 };

@@ -64,14 +64,27 @@ int fo_device_info(int* cu_count, int* clock_khz, int* xcd_count);
 /* D[M,N] = A[M,K] . B[N,K]^T, fp32 accumulate, natural row-major D.
  * Replaces gemm_func_table[Algo] / mutlass_gemm<TM,TN,TK>
  * (src/tiling/gemm_dispatcher.h:16-20, src/gemm/gemm.cu:29-113).
- * Requires M % BM == 0, N % BN == 0, K % 8 == 0 (a K that is not a multiple of 64
- * is zero-padded inside the kernel; the operands must then be below 2 GiB each), 16-byte aligned pointers. */
+ * Any M >= 1 and N >= 1 (the layout tile of `algo` places nothing here; rows
+ * and columns of an edge tile that lie outside the matrix are computed on
+ * zero-filled operand rows and not stored; an N that is not a multiple of 8
+ * makes the rows of D unaligned and is stored element by element), K % 8 == 0
+ * (a K that is not a multiple of 64 is zero-padded inside the kernel; the
+ * operands must then be below 2 GiB each), 16-byte aligned pointers.  The
+ * reference's kernels take only multiples of their tile (README.md:75; the
+ * residue predicates of src/overlap/gemm_with_signal.h:176-181 are never
+ * exercised by its callers). */
 int fo_gemm(int dtype, int algo, int M, int N, int K,
             const void* A, const void* B, void* D, void* stream);
 
 /* Signalling GEMM.  Tile t is stored at slot RA[t] of the permuted layout and,
- * after the tile's stores are visible device-wide, MM[group(slot)] is bumped
- * with a release-ordered atomic.  group(slot) is the index of the first
+ * after the tile's stores are visible device-wide, MM[group(slot)] is bumped.
+ * By default (fo_tune "release_mode" 1) the tile stores are agent-scope
+ * write-through stores; every wavefront waits until they are acknowledged,
+ * the workgroup meets at a barrier, and then one lane per group adds the
+ * group's tile count with a relaxed agent-scope atomic.  The release-ordered
+ * form (the atomic itself a release at agent scope, which writes the L2's
+ * dirty lines back first) is what "release_mode" 0 selects; counters, slots
+ * and results are the same.  group(slot) is the index of the first
  * inclusive prefix sum of cseg_dev[0..G) that exceeds slot.  If `monitor` is
  * non-zero a ticket is also taken from MM[TN-1] and stored at MM[TN+slot].
  * Replaces signal_func_table[Algo] / mutlass_gemm_signal<TM,TN,TK>
@@ -128,6 +141,8 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host);
 
 /* Process-wide tuning knobs of the GEMM epilogue, for measurement; no
  * counterpart in the reference.  Results are identical for every setting.
+ * The knobs are atomics: a thread may set one while others launch, and a
+ * launch reads each knob once.
  *   "release_mode" 1 (default): the tile stores are agent-scope write-through
  *                  stores; every wave waits for their acknowledgement, the
  *                  workgroup meets at a barrier, then a relaxed agent-scope
@@ -152,11 +167,14 @@ int fo_tune(const char* key, int value);
  * to *addr.  Replaces launch_kernel_wait_flag (src/wait_launch.h:5,
  * src/wait_launch.cu:5-7, kernel src/wait.cuh:5-9).  Unlike the reference the
  * wait is bounded (fo_set_wait_timeout_ms, default 10000 ms): on expiry the
- * kernel leaves *addr untouched, bumps the timeout count and returns; what
- * follows on the stream then works on an incomplete group, so a caller checks
- * fo_wait_timeouts at its next synchronisation point and zeroes MM after an
- * expiry. */
-int fo_wait(int that, int* addr, void* stream);
+ * kernel leaves *addr untouched, counts the expiry and returns; what follows
+ * on the stream then works on an incomplete group, so a caller reads the count
+ * at its next synchronisation point and zeroes MM after an expiry.
+ * `expired` (here and in the other waiting calls): a device int that the
+ * caller owns and that this call increments if its wait expires, so that a
+ * caller sees the expiries of its own calls only; NULL counts them in a word
+ * per device that fo_wait_timeouts reads. */
+int fo_wait(int that, int* addr, int* expired, void* stream);
 
 /* One persistent kernel in place of G (wait, collective) launch pairs: for
  * g = 0..G-1 in order, wait for MM[g] == cseg_dev[g], copy group g's
@@ -177,16 +195,18 @@ int fo_wait(int that, int* addr, void* stream);
  * released strictly in index order by the whole grid, smaller ones as they
  * complete.  order_log (optional, G ints) gets order_log[g] = g when group g
  * has been released and its counter reset.  If a wait expires the wavefront
- * counts it (fo_wait_timeouts) and stops; MM then holds partial counts and
- * must be zeroed by the caller before it is used again. */
+ * counts it (in *expired, or for NULL in the word fo_wait_timeouts reads) and
+ * stops; MM then holds partial counts and must be zeroed by the caller before
+ * it is used again. */
 int fo_wait_consume(const int* cseg_dev, int G, int* MM,
                     const void* src, void* dst, long long tile_elems,
                     int nslices, int slice_first, int slice_count, long long slice_stride,
-                    int* order_log, int nblocks, void* stream);
+                    int* order_log, int nblocks, int* expired, void* stream);
 
 int fo_set_wait_timeout_ms(int ms);
-/* Number of bounded waits that expired on the current device since the last
- * call with reset != 0 (synchronises the device). */
+/* Number of bounded waits that were given no `expired` word of their own and
+ * expired on the current device since the last call with reset != 0
+ * (synchronises the device). */
 int fo_wait_timeouts(int* count, int reset);
 
 /* Copy `bytes` bytes (multiple of 2) from src to dst with a device kernel: the
@@ -198,11 +218,11 @@ int fo_consume(const void* src, void* dst, size_t bytes, void* stream);
  * enqueued earlier on the same `stream`: stream order has already made the
  * counter final, so there is nothing to poll.  *addr == that is cleared to 0 as
  * fo_wait does; any other value is left in place and counted as an expired wait
- * (fo_wait_timeouts).  The copy is made either way, as it would be behind an
+ * (`expired` as in fo_wait).  The copy is made either way, as it would be behind an
  * expired fo_wait.  Used for the last group of a call, which completes together
  * with the GEMM (the reference waits for it on the communication stream,
  * src/overlap_impl.cu:257-265, and then joins the streams). */
-int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t bytes, void* stream);
+int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t bytes, int* expired, void* stream);
 
 /* One launch for the `nslices` slices of a released group: slice k is the
  * `slice_bytes` bytes at src + k * slice_bytes and goes to dst + k *
@@ -221,7 +241,7 @@ int fo_settle_consume(int that, int* addr, const void* src, void* dst, size_t by
 #define FO_COPY_STREAM 1
 #define FO_COPY_CACHED 2
 int fo_consume_slices(int that, int* addr, const void* src, void* dst, size_t slice_bytes, int nslices,
-                      size_t dst_stride_bytes, int store_policy, void* stream);
+                      size_t dst_stride_bytes, int store_policy, int* expired, void* stream);
 
 /* ---- RMSNorm ---------------------------------------------------------- */
 

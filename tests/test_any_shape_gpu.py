@@ -1,0 +1,108 @@
+"""Shapes the reference's kernels do not take (README.md:75 of the reference: "the GEMM size
+must be multiples of the tile"; src/rmsnorm/rmsnorm_launch.cu:11-21: rows of at most 1024 x 16
+elements): the plain GEMM for any M and N, RMSNorm and reorder+RMSNorm for rows longer than a
+wavefront keeps in registers.  All through the C ABI, against the oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from flashoverlap_amd import capi
+from oracle import fo_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_TOL, MAX_ABS_TOL = 1e-3, 2e-2     # the path's tolerance for floating-point results
+
+
+@pytest.fixture(scope="module")
+def L(fo_lib, dev):
+    return fo_lib
+
+
+GUARD = 4096   # elements in front of and behind D that no launch may touch
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [
+    (1000, 1160, 264),     # ragged in M and N (N a multiple of 8), partial last k panel
+    (1, 8, 8), (8, 1, 16), (3, 5, 24),           # smaller than any tile
+    (127, 129, 72), (130, 7, 64), (257, 255, 136),   # N not a multiple of 8: rows of D are unaligned
+    (300, 520, 1000), (129, 2048, 64), (2049, 136, 128),
+    (4100, 2056, 512),     # 256x256 macro tiles with ragged last row and column of tiles
+    (384, 640, 320),       # multiples of 128: the kernel without predicates
+])
+def test_plain_gemm_any_shape_bit_exact_on_integer_inputs(L, dev, dt, M, N, K):
+    print(f"any-shape gemm {dt} {M}x{N}x{K}", flush=True)
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K)
+    A = torch.randint(-2, 3, (M, K), generator=g).to(dt)
+    B = torch.randint(-2, 3, (N, K), generator=g).to(dt)
+    # operands allocated exactly: a read beyond them would land in whatever the allocator put next
+    dA, dB = A.to(dev), B.to(dev)
+    buf = torch.full((GUARD + M * N + GUARD,), 7.0, dtype=dt, device=dev)
+    D = buf[GUARD:GUARD + M * N]
+    assert D.data_ptr() % 16 == 0
+    for algo in (1, 3):    # the layout tile of `algo` places nothing in the plain GEMM
+        D.fill_(7.0)
+        capi.check(L.fo_gemm(capi.dtype_code(dt), algo, M, N, K, dA.data_ptr(), dB.data_ptr(), D.data_ptr(), None))
+        torch.cuda.synchronize()
+        assert torch.equal(D.cpu().view(M, N), O.gemm(A, B))
+        assert (buf[:GUARD] == 7.0).all() and (buf[GUARD + M * N:] == 7.0).all()
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_plain_gemm_any_shape_random_within_tolerance(L, dev, dt):
+    M, N, K = 1000, 1160, 2040
+    g = torch.Generator().manual_seed(9)
+    A = (torch.randn(M, K, generator=g) / K ** 0.5).to(dt)
+    B = (torch.randn(N, K, generator=g) / K ** 0.5).to(dt)
+    D = torch.empty(M, N, dtype=dt, device=dev)
+    dA, dB = A.to(dev), B.to(dev)
+    capi.check(L.fo_gemm(capi.dtype_code(dt), 1, M, N, K, dA.data_ptr(), dB.data_ptr(), D.data_ptr(), None))
+    torch.cuda.synchronize()
+    ref = O.gemm_fp32(A, B).to(dt)
+    assert O.rel_l2(D.cpu(), ref) < REL_L2_TOL and O.max_abs(D.cpu(), ref) < MAX_ABS_TOL
+    ulp = 2 ** -10 if dt == torch.float16 else 2 ** -7
+    assert ((D.cpu().float() - ref.float()).abs() <= ulp * ref.float().abs() + 1e-6).all()
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bs,dim", [(5, 16392), (3, 20480), (4, 32768), (2, 65544), (1, 131072)])
+def test_plain_rmsnorm_long_rows(L, dev, dt, bs, dim):
+    g = torch.Generator().manual_seed(dim)
+    x = torch.randn(bs, dim, generator=g).to(dt)
+    gamma = (1 + 0.1 * torch.randn(dim, generator=g)).to(dt)
+    buf = torch.full((GUARD + bs * dim + GUARD,), 7.0, dtype=dt, device=dev)
+    out = buf[GUARD:GUARD + bs * dim]
+    dx, dgamma = x.to(dev), gamma.to(dev)
+    capi.check(L.fo_rmsnorm(capi.dtype_code(dt), dx.data_ptr(), dgamma.data_ptr(), out.data_ptr(), bs, dim, 1e-5, None))
+    torch.cuda.synchronize()
+    ref = O.rmsnorm(x, gamma, 1e-5)
+    got = out.cpu().view(bs, dim)
+    assert O.rel_l2(got, ref) < REL_L2_TOL and O.max_abs(got, ref) < MAX_ABS_TOL
+    # two roundings in the reference's order: within two storage ulps of the oracle
+    ulp = 2 ** -10 if dt == torch.float16 else 2 ** -7
+    assert ((got.float() - ref.float()).abs() <= 2 * ulp * ref.float().abs() + 1e-6).all()
+    assert (buf[:GUARD] == 7.0).all() and (buf[GUARD + bs * dim:] == 7.0).all()
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bs,dim,BM,BN,rldn", [(256, 20480, 128, 128, 1), (128, 32768, 64, 256, 2), (32, 16640, 16, 128, 1)])
+def test_reorder_rmsnorm_long_rows(L, dev, dt, bs, dim, BM, BN, rldn):
+    g = torch.Generator().manual_seed(dim + BM)
+    Cn = torch.randn(bs, dim, generator=g).to(dt)
+    gamma = (1 + 0.1 * torch.randn(dim, generator=g)).to(dt)
+    T = (bs // BM) * (dim // BN)
+    ra = O.reorder_indices(T, np.random.default_rng(T).permutation(T))
+    x = O.place_tiles(Cn, ra, BM, BN, rldn)
+    out = torch.empty(bs, dim, dtype=dt, device=dev)
+    dx, dgamma, dra = x.to(dev), gamma.to(dev), torch.from_numpy(ra).to(dev)
+    capi.check(L.fo_reorder_rmsnorm(capi.dtype_code(dt), dx.data_ptr(), dgamma.data_ptr(), out.data_ptr(), bs, dim,
+                                    BM, BN, rldn, dra.data_ptr(), 1e-6, None))
+    torch.cuda.synchronize()
+    ref = O.reorder_rmsnorm(x, gamma, bs, dim, BM, BN, rldn, ra, 1e-6)
+    assert torch.equal(ref, O.rmsnorm(Cn, gamma, 1e-6))
+    assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and O.max_abs(out.cpu(), ref) < MAX_ABS_TOL
+    ulp = 2 ** -10 if dt == torch.float16 else 2 ** -7
+    assert ((out.cpu().float() - ref.float()).abs() <= 2 * ulp * ref.float().abs() + 1e-6).all()

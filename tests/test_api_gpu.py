@@ -27,11 +27,13 @@ def _overlap(api, rank=0, size=1):
     return o
 
 
-def _timeouts():
+def _timeouts(*objects):
+    """Expired waits: those counted in the words the given OverlapImpl objects own, plus those of
+    callers that passed no word of their own (the per-device count of the C ABI)."""
     import ctypes
     n = ctypes.c_int()
     capi.check(capi.lib().fo_wait_timeouts(ctypes.byref(n), 1))
-    return n.value
+    return n.value + sum(o.wait_timeouts(True) for o in objects)
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
@@ -84,7 +86,7 @@ def test_allreduce_overlap_like_correctness_ar(api, dev, mode):
         y = torch.empty(M, N, dtype=torch.float16, device=dev)
         torch.ops.flashoverlap_op.reorder_rmsnorm(o.staging().view(M, N), y, W, BM, BN, 1, RA)
         torch.cuda.synchronize()
-        assert _timeouts() == 0
+        assert _timeouts(o) == 0
         assert counter.cpu().sum() == 0
         cref = O.gemm(A, B)
         # placement bit-exact: the staging buffer is the plain GEMM of the same kernel, permuted by the oracle
@@ -124,7 +126,7 @@ def test_reducescatter_overlap_like_correctness_rs(api, dev, stacked):
     out = torch.zeros((ws, M // ws, N) if stacked else (M // ws, N), dtype=torch.bfloat16, device=dev)
     o.gemm_reducescatter_overlap(A0.to(dev), B.to(dev), tmp, out, counter, RA, RE, 1, cSeg_CPU, cSeg_GPU, algo, False)
     torch.cuda.synchronize()
-    assert _timeouts() == 0 and counter.cpu().sum() == 0
+    assert _timeouts(o) == 0 and counter.cpu().sum() == 0
     cref = O.gemm(A0, B)
     slices = O.consume_reducescatter(O.scatter_place(cref, RA.cpu().numpy(), RE.cpu().numpy(), BM, BN, 1), cseg, BM,
                                      BN, ws)
@@ -161,7 +163,7 @@ def test_monitor_pass_like_the_tuner(api, dev):
         o.gemm_allreduce_overlap(A, B, C, MonitoredMatrix, ReorderedArray, 1, cSeg_CPU, cSeg_CPU.to(dev), algo, True)
         samples[i, :] = MonitoredMatrix[1:, :].view(-1)
     torch.cuda.synchronize()
-    assert _timeouts() == 0
+    assert _timeouts(o) == 0
     for i in range(3):
         assert sorted(samples[i].cpu().tolist()) == list(range(T))
     assert MonitoredMatrix[0, TN - 1].item() == T
@@ -190,19 +192,20 @@ def test_api_argument_checks(api, dev):
     with pytest.raises(RuntimeError, match="more than one GPU"):
         _overlap(api, 0, 2).gemm_all2all(A, A, C, C, 1, torch.zeros(2, 2, dtype=torch.int32))
     torch.cuda.synchronize()
-    assert _timeouts() == 0
+    assert _timeouts(o) == 0
 
 
 def test_expired_wait_is_reported_through_the_torch_api(api, dev):
     """A wait bound far below the GEMM's run time (forced from the host; every kernel still exits
     normally): in checked mode the overlapped call raises, the counters come back zeroed, and the
     same object then runs a correct call."""
-    M, N, K, algo = 8192, 8192, 16384, 1
+    M, N, K, algo = 8192, 8192, 32768, 1
     BM, BN, _ = capi.algo_tile(algo)
     TM, TN = M // BM, N // BN
     T = TM * TN
     # two groups: the first one (released on the second stream, where the wait starts with the GEMM)
-    # holds tiles of the GEMM's last round, so it completes only when the GEMM ends, after ~1.5 ms
+    # holds tiles of the GEMM's last round, so it completes only when the GEMM ends: more than 2 ms
+    # even on constant operands at full clock (4.4 PFLOP of work), twice the 1 ms bound
     cSeg_CPU = torch.tensor([T - 256, 256], dtype=torch.int32)
     cSeg_GPU = cSeg_CPU.to(dev)
     counter = torch.zeros(TN, dtype=torch.int32, device=dev)
@@ -224,6 +227,52 @@ def test_expired_wait_is_reported_through_the_torch_api(api, dev):
     torch.cuda.synchronize()
     assert o.wait_timeouts(True) == 0 and counter.cpu().sum() == 0
     assert (o.staging() == K).all()
+
+
+def test_an_expired_wait_belongs_to_the_object_that_made_it(api, dev):
+    """Two OverlapImpl objects on one device.  The first runs, unchecked, a call whose wait is
+    forced to expire from the host (1 ms bound, a GEMM of more than 2 ms); the second, in checked
+    mode, then runs a small correct call.  The expiry is counted in the first object's own word:
+    the second neither raises nor has its counters cleared, reports no expiry, and the per-device
+    word of callers that pass no word of their own stays at zero."""
+    M, N, K, algo = 8192, 8192, 32768, 1
+    BM, BN, _ = capi.algo_tile(algo)
+    TM, TN = M // BM, N // BN
+    T = TM * TN
+    cSeg_CPU = torch.tensor([T - 256, 256], dtype=torch.int32)
+    counter = torch.zeros(TN, dtype=torch.int32, device=dev)
+    RA = tiling.reorder_indices(T, tiling.raster_hint(M, N, algo), dev).reshape(TM, TN)
+    A = torch.ones(M, K, dtype=torch.bfloat16, device=dev)
+    B = torch.ones(N, K, dtype=torch.bfloat16, device=dev)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    m, n, k = 512, 512, 256
+    tm, tn = m // BM, n // BN
+    cseg2 = torch.tensor([3, tm * tn - 3], dtype=torch.int32)
+    counter2 = torch.zeros(tn, dtype=torch.int32, device=dev)
+    ra2 = tiling.reorder_indices(tm * tn, tiling.raster_hint(m, n, algo), dev).reshape(tm, tn)
+    a2 = torch.ones(m, k, dtype=torch.bfloat16, device=dev)
+    b2 = torch.ones(n, k, dtype=torch.bfloat16, device=dev)
+    c2 = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    first, second = _overlap(api), _overlap(api)
+    second.set_check_timeouts(True)
+    assert _timeouts() == 0
+    first.set_wait_timeout_ms(1)          # process-wide: the small call below stays far inside it
+    try:
+        first.gemm_allreduce_overlap(A, B, C, counter, RA, 1, cSeg_CPU, cSeg_CPU.to(dev), algo, False)
+        torch.cuda.synchronize()
+        second.gemm_allreduce_overlap(a2, b2, c2, counter2, ra2, 1, cseg2, cseg2.to(dev), algo, False)   # must not raise
+    finally:
+        first.set_wait_timeout_ms(5000)
+    torch.cuda.synchronize()
+    assert second.wait_timeouts(False) == 0 and counter2.cpu().sum() == 0
+    assert (second.staging() == k).all()
+    assert first.wait_timeouts(True) == 1 and first.wait_timeouts(False) == 0
+    assert counter.cpu()[0] == T - 256    # the unchecked caller's counters are its own to clear
+    assert _timeouts() == 0
+    counter.zero_()
+    first.gemm_allreduce_overlap(A, B, C, counter, RA, 1, cSeg_CPU, cSeg_CPU.to(dev), algo, False)
+    torch.cuda.synchronize()
+    assert first.wait_timeouts(True) == 0 and counter.cpu().sum() == 0 and (first.staging() == K).all()
 
 
 def test_consumer_blocks_are_limited_to_the_cu_count(api, dev):

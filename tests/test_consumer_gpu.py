@@ -31,7 +31,7 @@ def test_ragged_groups(fo_lib, dev, nblocks, ws):
     log = torch.full((G,), -1, dtype=torch.int32, device=dev)
     stride = (T * BM * BN) // ws if ws > 1 else 0
     capi.check(L.fo_wait_consume(cs.data_ptr(), G, MM.data_ptr(), d_src.data_ptr(), d_dst.data_ptr(), BM * BN, ws, 0,
-                                 ws, stride, log.data_ptr(), nblocks, None))
+                                 ws, stride, log.data_ptr(), nblocks, None, None))
     torch.cuda.synchronize()
     n = C.c_int()
     capi.check(L.fo_wait_timeouts(C.byref(n), 1))
@@ -53,6 +53,6 @@ def test_more_workgroups_than_cus_is_refused(fo_lib, dev):
     capi.check(L.fo_device_info(C.byref(cu), None, None))
     buf = torch.zeros(4096, dtype=torch.int32, device=dev)
     rc = L.fo_wait_consume(buf.data_ptr(), 1, buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), 128, 1, 0, 1, 0, None,
-                           cu.value + 1, None)
+                           cu.value + 1, None, None)
     assert rc == capi.FO_ERR_LIMIT
     assert b"one workgroup per CU" in L.fo_last_error()

@@ -16,13 +16,6 @@ from flashoverlap_amd import capi, tiling
 pytestmark = pytest.mark.gpu
 
 
-def _timeouts():
-    import ctypes
-    n = ctypes.c_int()
-    capi.check(capi.lib().fo_wait_timeouts(ctypes.byref(n), 1))
-    return n.value
-
-
 @pytest.mark.parametrize("w,mode", [(16, 1), (4, 2)])   # 4 groups released one by one; 16 groups, persistent consumer
 def test_overlapped_call_replays_from_a_graph(dev, w, mode):
     flashoverlap_amd.load()
@@ -67,6 +60,16 @@ def test_overlapped_call_replays_from_a_graph(dev, w, mode):
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=side):
                 call()
+            # checked mode waits for the call's completion, which a capture forbids: refused up front,
+            # before anything is enqueued, with an error that says so (capture_error_mode: the failed
+            # capture must not poison the streams of the rest of the process)
+            o.set_check_timeouts(True)
+            refused = torch.cuda.CUDAGraph()
+            with pytest.raises(RuntimeError, match="set_check_timeouts"):
+                with torch.cuda.graph(refused, stream=side, capture_error_mode="thread_local"):
+                    call()
+            o.set_check_timeouts(False)
+            del refused
             for replay in range(4):
                 print(f"graph replay {replay} w={w} mode={mode}", flush=True)
                 a_new, b_new = operands()
@@ -82,7 +85,7 @@ def test_overlapped_call_replays_from_a_graph(dev, w, mode):
                 torch.cuda.synchronize()
                 graph.replay()
                 torch.cuda.synchronize()
-                assert _timeouts() == 0
+                assert o.wait_timeouts(True) == 0
                 assert counter.cpu().sum() == 0
                 assert torch.equal(o.staging(), want_staging)
                 assert torch.equal(y, want_y)

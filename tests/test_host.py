@@ -56,8 +56,10 @@ def test_algo_table_matches_reference_instances(fo_lib):
 
 def test_argument_errors_return_codes_not_exits(fo_lib):
     # shape / argument validation happens before any device call
-    rc = fo_lib.fo_gemm(capi.FO_F16, 1, 100, 128, 64, 16, 16, 16, None)
+    # the plain GEMM takes any M and N; the signalling modes only multiples of the layout tile
+    rc = fo_lib.fo_gemm_signal(capi.FO_F16, 1, 100, 128, 64, 1, 16, 1, None, 16, 16, 16, 16, 16, 0, None)
     assert rc == capi.FO_ERR_SHAPE and b"multiples" in fo_lib.fo_last_error()
+    assert fo_lib.fo_gemm(capi.FO_F16, 1, 0, 128, 64, 16, 16, 16, None) == capi.FO_ERR_SHAPE
     assert fo_lib.fo_gemm(capi.FO_F16, 1, 128, 128, 36, 16, 16, 16, None) == capi.FO_ERR_SHAPE
     assert fo_lib.fo_gemm(7, 1, 128, 128, 64, 16, 16, 16, None) == capi.FO_ERR_ARG
     assert fo_lib.fo_gemm(capi.FO_F16, 9, 128, 128, 64, 16, 16, 16, None) == capi.FO_ERR_ARG
@@ -65,16 +67,16 @@ def test_argument_errors_return_codes_not_exits(fo_lib):
     assert fo_lib.fo_gemm(capi.FO_F16, 1, 128, 128, 64, 8, 16, 16, None) == capi.FO_ERR_ARG  # misaligned
     assert fo_lib.fo_gemm_signal(capi.FO_F16, 1, 128, 128, 64, 1, None, 1, None, 16, 16, 16, None, None, 0,
                                  None) == capi.FO_ERR_ARG
-    assert fo_lib.fo_wait(1, None, None) == capi.FO_ERR_ARG
+    assert fo_lib.fo_wait(1, None, None, None) == capi.FO_ERR_ARG
     assert fo_lib.fo_consume(16, 16, 3, None) == capi.FO_ERR_ARG
     assert fo_lib.fo_consume(None, None, 0, None) == capi.FO_OK  # empty copy is a no-op
     assert fo_lib.fo_reorder_rmsnorm(capi.FO_F16, 16, 16, 16, 8, 60, 4, 4, 1, 16, 1e-5, None) == capi.FO_ERR_SHAPE
     assert fo_lib.fo_reorder_rmsnorm(capi.FO_F16, 16, 16, 16, 8, 64, 4, 8, 1, None, 1e-5, None) == capi.FO_ERR_ARG
     assert fo_lib.fo_rmsnorm(capi.FO_F16, 16, 16, 16, 0, 64, 1e-5, None) == capi.FO_OK  # zero rows
-    assert fo_lib.fo_rmsnorm(capi.FO_F16, 16, 16, 16, 4, 32768, 1e-5, None) == capi.FO_ERR_LIMIT
+    assert fo_lib.fo_rmsnorm(capi.FO_F16, 16, 16, 16, 4, 32764, 1e-5, None) == capi.FO_ERR_SHAPE   # dim % 8
     assert fo_lib.fo_set_wait_timeout_ms(0) == capi.FO_ERR_ARG
-    assert fo_lib.fo_wait_consume(16, 2, 16, 16, 16, 100, 1, 0, 1, 0, None, 4, None) == capi.FO_ERR_SHAPE
-    assert fo_lib.fo_wait_consume(16, 2, 16, 16, 16, 128, 2, 1, 2, 0, None, 4, None) == capi.FO_ERR_ARG
+    assert fo_lib.fo_wait_consume(16, 2, 16, 16, 16, 100, 1, 0, 1, 0, None, 4, None, None) == capi.FO_ERR_SHAPE
+    assert fo_lib.fo_wait_consume(16, 2, 16, 16, 16, 128, 2, 1, 2, 0, None, 4, None, None) == capi.FO_ERR_ARG
 
 
 # ---- rasterisation ---------------------------------------------------------

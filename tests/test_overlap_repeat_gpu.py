@@ -66,11 +66,11 @@ def test_many_overlapped_iterations(fo_lib, dev, mode, store, rel, scatter):
                                             0, None))
             if mode == "persistent":
                 capi.check(L.fo_wait_consume(cs.data_ptr(), G, MM.data_ptr(), Cp.data_ptr(), staging.data_ptr(),
-                                             BM * BN, 1, 0, 1, 0, None, 16, comm))
+                                             BM * BN, 1, 0, 1, 0, None, 16, None, comm))
             else:
                 acc = 0
                 for gi, n in enumerate(cseg):
-                    capi.check(L.fo_wait(n, MM.data_ptr() + 4 * gi, comm))
+                    capi.check(L.fo_wait(n, MM.data_ptr() + 4 * gi, None, comm))
                     capi.check(L.fo_consume(Cp.data_ptr() + 2 * acc, staging.data_ptr() + 2 * acc, 2 * n * BM * BN,
                                             comm))
                     acc += n * BM * BN

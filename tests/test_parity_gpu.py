@@ -189,6 +189,16 @@ def test_time_next_launch_gives_the_kernel_duration(L, dev):
     assert 0 < t_in.value <= t_out.value
     assert flops / (t_in.value * 1e-3) < 2.6e15          # not faster than the chip
     assert L.fo_time_next_launch(inner0, None) == capi.FO_ERR_ARG
+    # a call that is rejected uses the pair up too: it must not stay armed for a later, unrelated launch
+    capi.check(L.fo_event_record(inner0, None))
+    capi.check(L.fo_event_record(inner1, None))
+    torch.cuda.synchronize()
+    capi.check(L.fo_time_next_launch(inner0, inner1))
+    assert L.fo_gemm(p.code, 1, 2048, 2048, 12, p.dA.data_ptr(), p.dB.data_ptr(), out.data_ptr(), None) == capi.FO_ERR_SHAPE
+    p.gemm_plain(out=out)                      # 30 us of kernel that the pair must not see
+    torch.cuda.synchronize()
+    capi.check(L.fo_event_elapsed_ms(inner0, inner1, C.byref(t_in)))
+    assert t_in.value < 0.01, "the pair of a rejected call was attached to the next launch"
     for e in evs:
         capi.check(L.fo_event_destroy(e))
 
@@ -242,7 +252,12 @@ def test_mfma_spin_runs_counts_its_work_and_leaves_the_sink_alone(L, dev, dt, wi
 def test_gemm_rejects_unsupported_shapes(L, dev):
     a = torch.zeros(384, 384, dtype=torch.float16, device=dev)  # large enough for every call below
     assert L.fo_gemm(capi.FO_F16, 1, 256, 256, 44, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
-    assert L.fo_gemm(capi.FO_F16, 3, 384, 384, 64, a.data_ptr(), a.data_ptr(), a.data_ptr(), None) == capi.FO_ERR_SHAPE
+    # the signalling modes place whole layout tiles (128x256 here); the plain GEMM takes the shape
+    i = torch.zeros(64, dtype=torch.int32, device=dev)
+    assert L.fo_gemm_signal(capi.FO_F16, 3, 384, 384, 64, 1, i.data_ptr(), 1, None, a.data_ptr(), a.data_ptr(),
+                            a.data_ptr(), i.data_ptr(), i.data_ptr(), 0, None) == capi.FO_ERR_SHAPE
+    capi.check(L.fo_gemm(capi.FO_F16, 3, 384, 384, 64, a.data_ptr(), a.data_ptr(), a.data_ptr(), None))
+    torch.cuda.synchronize()
 
 
 # ---- signalling epilogue -------------------------------------------------------
@@ -392,7 +407,7 @@ def test_scatter_epilogue_and_reducescatter_slices(L, dev, comm_stream, ws, cseg
     # consumer: all ws receive buffers side by side
     D = torch.zeros(ws, M * N // ws, dtype=p.dt, device=dev)
     capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), D.data_ptr(), BM * BN,
-                                 ws, 0, ws, M * N // ws, None, 4, comm_stream))
+                                 ws, 0, ws, M * N // ws, None, 4, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert _timeouts(L) == 0
     assert torch.equal(D.cpu(), O.consume_reducescatter(want, cseg, BM, BN, ws))
@@ -408,7 +423,7 @@ def test_scatter_epilogue_and_reducescatter_slices(L, dev, comm_stream, ws, cseg
     p.gemm_signal()
     one = torch.zeros(M * N // ws, dtype=p.dt, device=dev)
     capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), one.data_ptr(), BM * BN,
-                                 ws, 1, 1, 0, None, 2, comm_stream))
+                                 ws, 1, 1, 0, None, 2, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert torch.equal(one.cpu(), O.consume_reducescatter(want, cseg, BM, BN, ws)[1])
 
@@ -523,14 +538,14 @@ def test_random_shapes_scatter_bit_exact(L, dev, seed):
 
 def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
     mm = torch.tensor([3, 9], dtype=torch.int32, device=dev)
-    capi.check(L.fo_wait(3, mm.data_ptr(), comm_stream))
+    capi.check(L.fo_wait(3, mm.data_ptr(), None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert mm.cpu().tolist() == [0, 9] and _timeouts(L) == 0
     # a count that is never reached: the waiter gives up after the limit, leaves
     # the counter alone and the stream carries on (the reference would spin forever)
     capi.check(L.fo_set_wait_timeout_ms(50))
     try:
-        capi.check(L.fo_wait(5, mm.data_ptr() + 4, comm_stream))
+        capi.check(L.fo_wait(5, mm.data_ptr() + 4, None, comm_stream))
         capi.check(L.fo_stream_sync(comm_stream))
         assert mm.cpu().tolist() == [0, 9] and _timeouts(L) == 1
         src = torch.arange(4096, dtype=torch.int16, device=dev)
@@ -538,7 +553,7 @@ def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
         bad = torch.tensor([1, 1], dtype=torch.int32, device=dev)
         flags = torch.tensor([1, 0], dtype=torch.int32, device=dev)   # group 1 never completes
         capi.check(L.fo_wait_consume(bad.data_ptr(), 2, flags.data_ptr(), src.data_ptr(), dst.data_ptr(), 2048, 1, 0,
-                                     1, 0, None, 3, comm_stream))
+                                     1, 0, None, 3, None, comm_stream))
         capi.check(L.fo_stream_sync(comm_stream))
         assert _timeouts(L) == 1                      # the one workgroup that owns the small group reports and leaves
         assert torch.equal(dst[:2048], src[:2048]) and not dst[2048:].any()
@@ -552,19 +567,19 @@ def test_settle_consume_clears_the_right_count_and_reports_a_wrong_one(L, dev, c
     mm = torch.tensor([7, 9, 0], dtype=torch.int32, device=dev)
     src = torch.randint(-30000, 30000, (40000,), dtype=torch.int16, device=dev)
     dst = torch.zeros_like(src)
-    capi.check(L.fo_settle_consume(7, mm.data_ptr(), src.data_ptr(), dst.data_ptr(), 2 * 40000, comm_stream))
+    capi.check(L.fo_settle_consume(7, mm.data_ptr(), src.data_ptr(), dst.data_ptr(), 2 * 40000, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 0 and torch.equal(dst, src)
     # a wrong count stays where it is and is counted, at once (no polling); the copy is still made
     dst.zero_()
-    capi.check(L.fo_settle_consume(8, mm.data_ptr() + 4, src.data_ptr(), dst.data_ptr(), 2 * 40000, comm_stream))
+    capi.check(L.fo_settle_consume(8, mm.data_ptr() + 4, src.data_ptr(), dst.data_ptr(), 2 * 40000, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 1 and torch.equal(dst, src)
     # an empty group still settles its counter
-    capi.check(L.fo_settle_consume(0, mm.data_ptr() + 8, src.data_ptr(), dst.data_ptr(), 0, comm_stream))
+    capi.check(L.fo_settle_consume(0, mm.data_ptr() + 8, src.data_ptr(), dst.data_ptr(), 0, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 0
-    assert L.fo_settle_consume(0, None, src.data_ptr(), dst.data_ptr(), 16, comm_stream) == capi.FO_ERR_ARG
+    assert L.fo_settle_consume(0, None, src.data_ptr(), dst.data_ptr(), 16, None, comm_stream) == capi.FO_ERR_ARG
 
 
 def test_consume_slices_equals_one_copy_per_slice(L, dev, comm_stream):
@@ -578,7 +593,7 @@ def test_consume_slices_equals_one_copy_per_slice(L, dev, comm_stream):
         capi.check(L.fo_consume(src.data_ptr() + 2 * (64 + k * part), want.data_ptr() + 2 * k * stride, 2 * part,
                                 comm_stream))
     capi.check(L.fo_consume_slices(0, None, src.data_ptr() + 2 * 64, got.data_ptr(), 2 * part, ws, 2 * stride,
-                                   capi.FO_COPY_STREAM, comm_stream))
+                                   capi.FO_COPY_STREAM, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert torch.equal(got, want)
     assert (got.view(ws, stride)[:, part:] == -1).all()      # nothing written between the slices
@@ -586,13 +601,13 @@ def test_consume_slices_equals_one_copy_per_slice(L, dev, comm_stream):
     mm = torch.tensor([5], dtype=torch.int32, device=dev)
     got.fill_(-1)
     capi.check(L.fo_consume_slices(5, mm.data_ptr(), src.data_ptr() + 2 * 64, got.data_ptr(), 2 * part, ws, 2 * stride,
-                                   capi.FO_COPY_CACHED, comm_stream))
+                                   capi.FO_COPY_CACHED, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert torch.equal(got, want) and mm.item() == 0 and _timeouts(L) == 0
     # slices that are not whole 16-byte units are refused
-    assert L.fo_consume_slices(0, None, src.data_ptr(), got.data_ptr(), 2 * 4100, 2, 2 * stride, capi.FO_COPY_AUTO,
+    assert L.fo_consume_slices(0, None, src.data_ptr(), got.data_ptr(), 2 * 4100, 2, 2 * stride, capi.FO_COPY_AUTO, None,
                                comm_stream) == capi.FO_ERR_SHAPE
-    assert L.fo_consume_slices(0, None, src.data_ptr(), got.data_ptr(), 2 * 4096, 2, 2 * stride, 7,
+    assert L.fo_consume_slices(0, None, src.data_ptr(), got.data_ptr(), 2 * 4096, 2, 2 * stride, 7, None,
                                comm_stream) == capi.FO_ERR_ARG
 
 
@@ -628,11 +643,11 @@ def test_overlapped_release_order_and_staging(L, dev, comm_stream, mode):
         p.gemm_signal()
         if mode == "persistent":
             capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(),
-                                         staging.data_ptr(), BM * BN, 1, 0, 1, 0, log.data_ptr(), 6, comm_stream))
+                                         staging.data_ptr(), BM * BN, 1, 0, 1, 0, log.data_ptr(), 6, None, comm_stream))
         else:
             acc = 0
             for g, n in enumerate(cseg):
-                capi.check(L.fo_wait(n, p.dMM.data_ptr() + 4 * g, comm_stream))
+                capi.check(L.fo_wait(n, p.dMM.data_ptr() + 4 * g, None, comm_stream))
                 capi.check(L.fo_consume(p.dC.data_ptr() + 2 * acc, staging.data_ptr() + 2 * acc, 2 * n * BM * BN,
                                         comm_stream))
                 acc += n * BM * BN
@@ -706,7 +721,7 @@ def _full_path(L, dev, comm_stream, dt, M, N, K, w, eps, ws=1, a_std=None, b_std
     dst = torch.zeros(M * N, dtype=dt, device=dev)
     p.gemm_signal()
     capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), dst.data_ptr(), BM * BN,
-                                 ws, 0, ws, M * N // ws if ws > 1 else 0, None, 8, comm_stream))
+                                 ws, 0, ws, M * N // ws if ws > 1 else 0, None, 8, None, comm_stream))
     capi.check(L.fo_stream_join(comm_stream, None))
     torch.cuda.synchronize()
     assert _timeouts(L) == 0
