@@ -12,8 +12,6 @@ struct Knobs {
     std::atomic<int> store_mode{1};             // 0 = cached tile stores, 1 = agent-scope write-through stores (sc1)
     std::atomic<int> release_mode{1};           // 1 = write-through tile stores, acknowledged, then a relaxed atomic; 0 = release-ordered atomic
     std::atomic<int> copy_streaming_stores{2};  // consumer copies: 0 ordinary stores, 1 non-temporal, 2 chosen per launch
-    std::atomic<int> consumer_poll{0};          // persistent consumer: 0 = every wavefront polls its groups, 1 = one poller per workgroup
-    std::atomic<int> poll_nap{0};
     std::atomic<int> wait_timeout_ms{10000};    // bound of every device-side wait
 };
 
@@ -31,8 +29,6 @@ inline bool set_knob(std::string_view key, int value) {
     else if (key == "release_mode") k.release_mode.store(value ? 1 : 0, std::memory_order_relaxed);
     else if (key == "copy_streaming_stores" && value >= 0 && value <= 2)
         k.copy_streaming_stores.store(value, std::memory_order_relaxed);
-    else if (key == "poll_nap") k.poll_nap.store(value, std::memory_order_relaxed);
-    else if (key == "consumer_poll") k.consumer_poll.store(value ? 1 : 0, std::memory_order_relaxed);
     else return false;
     return true;
 }

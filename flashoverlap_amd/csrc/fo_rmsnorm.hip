@@ -39,26 +39,18 @@ struct Vec8<__bf16> {
 constexpr int kRowsPerBlock = 4;  // one wavefront per row; neighbouring rows read neighbouring tile segments
 constexpr int kWideThreads = 256;  // rows too long for one wavefront's registers: one workgroup per row
 
+// Ordinary loads, streaming (non-temporal) stores: the result is not read again here, and it
+// must not displace the GEMM operands held in the memory-side cache.  Measured on 8192 x 4096
+// against this choice: non-temporal loads 26 us instead of 20 over rotating buffers, ordinary
+// stores 28; the other cache-policy bits on the stores (sc1, sc0 sc1, with and without nt) equal
+// or slower.
 template <typename V>
 __device__ __forceinline__ V load_row_chunk(const V* p) {
-#ifdef FO_RMS_LOAD_NT
-    return __builtin_nontemporal_load(p);
-#else
     return *p;
-#endif
 }
-// streaming store by default: the result is not read again here, and it must not displace the
-// GEMM operands held in the memory-side cache
 template <typename V>
 __device__ __forceinline__ void store_row_chunk(V v, V* p) {
-#if defined(FO_RMS_STORE_BITS)
-    typedef unsigned int lab_u32x4 __attribute__((ext_vector_type(4)));
-    asm volatile("global_store_dwordx4 %0, %1, off " FO_RMS_STORE_BITS ::"v"(p), "v"(__builtin_bit_cast(lab_u32x4, v)) : "memory");
-#elif defined(FO_RMS_STORE_PLAIN)
-    *p = v;
-#else
     __builtin_nontemporal_store(v, p);
-#endif
 }
 
 enum { kNormPlain = 0, kNormGather = 1, kNormGatherFast = 2 };

@@ -33,17 +33,16 @@ __device__ int g_wait_timeouts = 0;
 __device__ __forceinline__ void count_expired(int* expired) { atomicAdd(expired ? expired : &g_wait_timeouts, 1); }
 
 // Bounded poll of *addr until pred(value); returns false on expiry.
+// long_naps: 127 x 64 clocks (about 3 us) between two looks instead of 8 x 64 (0.2 us).
 template <typename Pred>
-__device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, Pred pred, int nap = 0) {
+__device__ __forceinline__ bool bounded_poll(const int* addr, long long ticks, Pred pred, bool long_naps = false) {
     const long long t0 = wall_clock64();
     for (;;) {
         const int v = __hip_atomic_load(addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (pred(v)) return true;
         if (wall_clock64() - t0 > ticks) return false;
-        if (nap <= 0) __builtin_amdgcn_s_sleep(8);
-        else if (nap == 1) __builtin_amdgcn_s_sleep(32);
-        else
-            for (int i = 0; i < (nap >= 4 ? 4 : nap >= 3 ? 2 : 1); ++i) __builtin_amdgcn_s_sleep(127);
+        if (long_naps) __builtin_amdgcn_s_sleep(127);
+        else __builtin_amdgcn_s_sleep(8);
     }
 }
 
@@ -63,7 +62,7 @@ __global__ void wait_kernel(int that, int* addr, long long ticks, int* expired) 
 constexpr int kCopyThreads = 512;  // workgroup size of the per-group copy kernel
 constexpr int kCopyUnroll = 8;     // 16-byte units in flight per thread
 constexpr int kWavesPerBlock = 4;  // persistent consumer: one wavefront per SIMD
-constexpr long long kUnitsPerMember = 2048;  // 32 KiB: what one wavefront takes of a group before another joins
+constexpr long long kUnitsPerMember = 8192;  // 128 KiB: what one workgroup takes of a group before another joins
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
@@ -109,43 +108,46 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
 
 // Persistent form of the host loop in src/overlap_impl.cu:257-265 (and
 // :312-323 for the ReduceScatter receive layout).  The members of the kernel
-// are its wavefronts; every member walks the groups in index order.  A group
-// is handled by a team of members whose size grows with the group (one member
-// per 32 KiB, at most all of them); the teams of consecutive groups are
-// consecutive windows of the member list, so many small groups are spread over
-// the members and one large group is copied by all of them.  A member waits
-// for the group's count, bumps MM[g] once more (the member that brings it to
-// cSeg[g] + team is the last to have seen the count and stores the 0) and
-// copies its stripe of the range.  With every member on every group the groups
-// are released strictly in index order; smaller teams release groups as they
-// complete.  A group's range is cut into nslices equal parts; parts
-// slice_first .. slice_first+slice_count-1 are copied, part k to
+// are its workgroups (four wavefronts each); every member walks the groups in
+// index order.  A group is handled by a team of members whose size grows with
+// the group (one member per 128 KiB, at most all of them); the teams of
+// consecutive groups are consecutive windows of the member list, so many small
+// groups are spread over the members and one large group is copied by all of
+// them.  A member waits for the group's count, bumps MM[g] once more (the
+// member that brings it to cSeg[g] + team is the last to have seen the count
+// and stores the 0) and copies its stripe of the range.  With every member on
+// every group the groups are released strictly in index order; smaller teams
+// release groups as they complete.  A group's range is cut into nslices equal
+// parts; parts slice_first .. slice_first+slice_count-1 are copied, part k to
 // dst + (k - slice_first)*stride + offset/nslices (the receive layout of a
 // ReduceScatter; nslices = 1 is the plain copy).
 //
 // The kernel uses no LDS and few registers: the GEMM workgroup that runs on the
 // same CU owns all of its LDS and most of its registers, and these wavefronts
-// have to fit beside it.  Each wavefront finds
-// its groups on its own: 64 groups at a time, one per lane, with wavefront
-// scans for the group offsets and the team windows.
-//
-// BY_WG: the members are the workgroups instead of the wavefronts (a team then has one workgroup
-// per 128 KiB of the group).  Only the first wavefront of a member polls; the other three wait at
-// a workgroup barrier, which costs the SIMDs they share with the GEMM no issue slots and the
-// memory system a quarter of the polls.  The barrier needs no LDS.  The poller's result cannot
-// be handed to the other wavefronts without LDS, so after an expired wait the workgroup goes
-// on: it copies the incomplete group (as the copy behind an expired wait kernel does) and polls
-// every later group just once.
-template <bool STREAM, bool BY_WG>
+// have to fit beside it.  Each wavefront finds the member's groups on its own
+// (64 groups at a time, one per lane, with wavefront scans for the group
+// offsets and the team windows), so the four wavefronts agree without
+// exchanging anything.  Only the first wavefront of a member polls; the other
+// three wait at a workgroup barrier (which needs no LDS), where they cost the
+// SIMDs they share with the GEMM no issue slots and the memory system no
+// polls.  Every wavefront polling its own groups, with short naps, cost the
+// GEMM beside it 13 % on 4096 groups of 64 KiB; this form costs it 6-7 %.
+// The poller naps long (3 us) between two looks at a counter, except on the
+// groups at the end of the list, each member's last: there the time to notice
+// is no longer hidden behind later groups and adds to the call.  The poller's
+// result cannot be handed to the other wavefronts without LDS, so after an
+// expired wait the workgroup goes on: it copies the incomplete group (as the
+// copy behind an expired wait kernel does) and looks at every later counter
+// just once.
+template <bool STREAM>
 __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
     const int* __restrict__ cseg, int G, int* MM, const uint4* __restrict__ src, uint4* __restrict__ dst,
     long long tile_units, int nslices, int slice_first, int slice_count, long long slice_stride_units,
-    int* order_log, long long ticks, int* expired, int nap) {
+    int* order_log, long long ticks, int* expired) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int self = BY_WG ? (int)blockIdx.x : (int)blockIdx.x * kWavesPerBlock + wave;
-    const int members = BY_WG ? (int)gridDim.x : (int)gridDim.x * kWavesPerBlock;
-    constexpr long long kPerMember = BY_WG ? kUnitsPerMember * kWavesPerBlock : kUnitsPerMember;
+    const int self = (int)blockIdx.x;
+    const int members = (int)gridDim.x;
     long long lo_base = 0;  // first 16-byte unit of the chunk's first group
     int start_base = 0;     // first member of that group's team
     for (int g0 = 0; g0 < G; g0 += 64) {
@@ -154,7 +156,7 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
         const long long units = tile_units * count;
         int team = 0;
         if (g < G) {
-            const long long want = (units + kPerMember - 1) / kPerMember;
+            const long long want = (units + kUnitsPerMember - 1) / kUnitsPerMember;
             team = (int)(want < 1 ? 1 : (want > members ? members : want));
         }
         // inclusive scans of units and team sizes over the 64 groups of the chunk
@@ -174,17 +176,17 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
         int me = self - start;   // the team is a window of the member list
         if (me < 0) me += members;
         unsigned long long mine = __ballot(g < G && me < team);
-        while (mine) {   // wave-uniform: the groups this wavefront belongs to, in index order
+        while (mine) {   // uniform over the workgroup: the groups this member belongs to, in index order
             const int b = __builtin_ctzll(mine);
             mine &= mine - 1;
             const int gg = g0 + b;
             const int tm = __shfl(team, b, 64), mem = __shfl(me, b, 64), need = __shfl(count, b, 64);
             const long long glo = __shfl(lo, b, 64);
-            int ok = 0;
-            if (lane == 0 && (!BY_WG || wave == 0)) {
-                ok = bounded_poll(MM + gg, ticks, [need](int v) { return v >= need; }, nap) ? 1 : 0;
-                if (!ok) {
+            if (wave == 0 && lane == 0) {
+                const bool long_naps = gg + members < G;   // not among the last groups of the list
+                if (!bounded_poll(MM + gg, ticks, [need](int v) { return v >= need; }, long_naps)) {
                     count_expired(expired);
+                    ticks = -1;   // every later poll looks once and gives up
                 } else {
                     // Every member has seen the full count once it has bumped it; the last one
                     // to do so puts the counter back.  The copies need not be finished for that:
@@ -199,20 +201,12 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
                     }
                 }
             }
+            __builtin_amdgcn_s_barrier();   // the three other wavefronts slept here
             const long long part = tile_units * need / nslices;
-            if constexpr (BY_WG) {
-                if (wave == 0 && !__shfl(ok, 0, 64)) ticks = -1;   // every later poll looks once and gives up
-                __builtin_amdgcn_s_barrier();                       // the three other wavefronts slept here
-                for (int k = 0; k < slice_count; ++k)
-                    team_copy<true, 64 * kWavesPerBlock, STREAM>(src + glo + (slice_first + k) * part,
-                                                                 dst + k * slice_stride_units + glo / nslices, part, mem,
-                                                                 tm, (int)threadIdx.x);
-            } else {
-                if (!__shfl(ok, 0, 64)) return;  // the wait expired: this wavefront gives up on the rest
-                for (int k = 0; k < slice_count; ++k)
-                    team_copy<true, 64, STREAM>(src + glo + (slice_first + k) * part,
-                                                dst + k * slice_stride_units + glo / nslices, part, mem, tm, lane);
-            }
+            for (int k = 0; k < slice_count; ++k)
+                team_copy<true, 64 * kWavesPerBlock, STREAM>(src + glo + (slice_first + k) * part,
+                                                             dst + k * slice_stride_units + glo / nslices, part, mem, tm,
+                                                             (int)threadIdx.x);
         }
         lo_base += __shfl(su, 63, 64);
         start_base = (int)(((long long)start_base + __shfl(st, 63, 64)) % members);
@@ -346,13 +340,10 @@ int launch_wait_consume(const int* cseg, int G, int* MM, const void* src, void* 
         return fail(FO_ERR_LIMIT, "fo_wait_consume: nblocks=%d outside 1..%d (one workgroup per CU)", nblocks, facts->cus);
     long long ticks;
     if (int e = ticks_for_timeout(&ticks)) return e;
-    const bool streaming = knob(knobs().copy_streaming_stores) != 0;   // it runs beside the GEMM
-    const bool by_wg = knob(knobs().consumer_poll) != 0;
-    auto kern = by_wg ? (streaming ? wait_consume_kernel<true, true> : wait_consume_kernel<false, true>)
-                      : (streaming ? wait_consume_kernel<true, false> : wait_consume_kernel<false, false>);
+    auto kern = knob(knobs().copy_streaming_stores) ? wait_consume_kernel<true> : wait_consume_kernel<false>;   // it runs beside the GEMM
     hipLaunchKernelGGL(kern, dim3(nblocks), dim3(64 * kWavesPerBlock), 0, stream, cseg, G, MM, (const uint4*)src,
                        (uint4*)dst, tile_elems / 8, nslices, slice_first, slice_count, slice_stride / 8, order_log, ticks,
-                       expired, knob(knobs().poll_nap));
+                       expired);
     FO_HIP(hipGetLastError());
     return FO_OK;
 }

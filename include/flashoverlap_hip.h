@@ -189,15 +189,18 @@ int fo_wait(int that, int* addr, int* expired, void* stream);
  * with all slices it is every rank's receive buffer side by side.
  * The kernel runs nblocks workgroups of four wavefronts (1 <= nblocks <= CU
  * count; it uses no LDS and few registers, so a workgroup fits beside a GEMM
- * workgroup on a CU).  Of the 4 * nblocks wavefronts a team of one per 32 KiB
- * of the group (at most all) handles a group; consecutive groups go to
- * consecutive teams.  Groups of nblocks x 128 KiB and more are therefore
+ * workgroup on a CU).  A team of workgroups, one per 128 KiB of the group (at
+ * most all), handles a group: its first wavefronts poll the counter, the
+ * others sleep at a barrier until it is full, then all copy.  Consecutive
+ * groups go to consecutive teams.  Groups of nblocks x 128 KiB and more are therefore
  * released strictly in index order by the whole grid, smaller ones as they
  * complete.  order_log (optional, G ints) gets order_log[g] = g when group g
- * has been released and its counter reset.  If a wait expires the wavefront
- * counts it (in *expired, or for NULL in the word fo_wait_timeouts reads) and
- * stops; MM then holds partial counts and must be zeroed by the caller before
- * it is used again. */
+ * has been released and its counter reset.  If a wait expires the workgroup
+ * counts it (in *expired, or for NULL in the word fo_wait_timeouts reads),
+ * copies the incomplete group like the copy behind an expired fo_wait would,
+ * and from then on looks at each of its later counters just once; MM then
+ * holds partial counts and must be zeroed by the caller before it is used
+ * again. */
 int fo_wait_consume(const int* cseg_dev, int G, int* MM,
                     const void* src, void* dst, long long tile_elems,
                     int nslices, int slice_first, int slice_count, long long slice_stride,

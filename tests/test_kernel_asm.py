@@ -129,6 +129,6 @@ def test_consumer_copy_variants_differ_in_their_stores(tmp_path):
             name = None
         if name and "global_store_dwordx4" in line:
             stores[name][1 if re.search(r"\bnt\b", line.split(";")[0]) else 2] += 1
-    assert len(stores) == 6   # consume_kernel x 2, wait_consume_kernel x 2 store policies x 2 polling forms
+    assert len(stores) == 4
     for name, (stream, nt, plain) in stores.items():
         assert (nt > 0 and plain == 0) if stream else (plain > 0 and nt == 0), (name, nt, plain)
