@@ -66,12 +66,10 @@ constexpr long long kUnitsPerMember = 8192;  // 128 KiB: what one workgroup take
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// Copies n 16-byte units (n * 16 < 4 GiB) as member `me` of a team of `team`
-// members of WIDTH threads each (`t` is the thread's index inside its member),
-// which interleave in chunks of WIDTH * kCopyUnroll units, every thread keeping
-// kCopyUnroll loads in flight.  COHERENT: read with agent-scope loads that do
-// not hit in the non-coherent caches (for data another XCD wrote while this
-// kernel runs).  The loads are non-temporal: the source streams through once.
+// Copies n 16-byte units as member `me` of a team of `team` members of WIDTH
+// threads each (`t` is the thread's index inside its member), which interleave
+// in chunks of WIDTH * kCopyUnroll units, every thread keeping kCopyUnroll
+// loads in flight.  The loads are non-temporal: the source streams through once.
 // STREAM: the stores are non-temporal too, which keeps the copy from displacing
 // the operands of a GEMM running beside it from the 256 MB memory-side cache
 // (with ordinary stores an overlapped 16384x8192x1024 GEMM ran 4 % longer);
@@ -79,21 +77,16 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // it next (reorder+RMSNorm right behind a copy took 25 us instead of 31).  A
 // compile-time choice: as a run-time branch around the two kinds of store the
 // compiler merges them into one ordinary store.
-template <bool COHERENT, int WIDTH, bool STREAM>
+template <int WIDTH, bool STREAM>
 __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __restrict__ d, long long n, int me,
                                           int team, int t) {
     const long long chunk = (long long)WIDTH * kCopyUnroll;
-    [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc;
-    if constexpr (COHERENT) rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, 0xffffffff, 0x00020000);
     for (long long base = (long long)me * chunk; base < n; base += (long long)team * chunk) {
         u32x4 v[kCopyUnroll];
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
             const long long i = base + u * WIDTH + t;
-            if (i < n) {
-                if constexpr (COHERENT) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(i * 16), 0, 16 | 2);  // sc1 nt
-                else v[u] = __builtin_nontemporal_load((const u32x4*)(s + i));
-            }
+            if (i < n) v[u] = __builtin_nontemporal_load((const u32x4*)(s + i));
         }
 #pragma unroll
         for (int u = 0; u < kCopyUnroll; ++u) {
@@ -103,6 +96,30 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
                 else *(u32x4*)(d + i) = v[u];
             }
         }
+    }
+}
+
+// The same for the persistent consumer, which runs beside the GEMM and has to live in the 64
+// registers that fit beside the GEMM's wavefront on a SIMD: the source is read with agent-scope
+// loads that do not hit in the non-coherent caches (another XCD wrote it while this kernel runs),
+// four units in flight per thread, source and destination addressed through buffer descriptors
+// with 32-bit offsets (n * 16 < 4 GiB) instead of a 64-bit pointer per access.
+constexpr int kCoherentUnroll = 4;
+template <int WIDTH, bool STREAM>
+__device__ __forceinline__ void team_copy_coherent(const uint4* __restrict__ s, uint4* __restrict__ d, unsigned n,
+                                                   unsigned me, unsigned team, unsigned t) {
+    constexpr unsigned chunk = WIDTH * kCoherentUnroll;
+    const __amdgpu_buffer_rsrc_t src = __builtin_amdgcn_make_buffer_rsrc((void*)s, 0, (int)(n * 16u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t dst = __builtin_amdgcn_make_buffer_rsrc((void*)d, 0, (int)(n * 16u), 0x00020000);
+    for (unsigned base = me * chunk; base < n; base += team * chunk) {
+        u32x4 v[kCoherentUnroll];
+        // a unit beyond n lies beyond the descriptors: it reads as zero and is not stored
+#pragma unroll
+        for (int u = 0; u < kCoherentUnroll; ++u)
+            v[u] = __builtin_amdgcn_raw_buffer_load_b128(src, (int)((base + u * WIDTH + t) * 16u), 0, 16 | 2);   // sc1 nt
+#pragma unroll
+        for (int u = 0; u < kCoherentUnroll; ++u)
+            __builtin_amdgcn_raw_buffer_store_b128(v[u], dst, (int)((base + u * WIDTH + t) * 16u), 0, STREAM ? 2 : 0);   // nt or not
     }
 }
 
@@ -139,8 +156,11 @@ __device__ __forceinline__ void team_copy(const uint4* __restrict__ s, uint4* __
 // expired wait the workgroup goes on: it copies the incomplete group (as the
 // copy behind an expired wait kernel does) and looks at every later counter
 // just once.
+// (At most 72 registers: the GEMM's wavefront on the same SIMD takes up to 440 of the 512.  A
+// consumer that needs more would, once resident, keep the GEMM's workgroup from being placed on
+// its CU, and then wait for that GEMM's signals until its waits expire.)
 template <bool STREAM>
-__global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
+__global__ void __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_per_eu(7, 8))) wait_consume_kernel(
     const int* __restrict__ cseg, int G, int* MM, const uint4* __restrict__ src, uint4* __restrict__ dst,
     long long tile_units, int nslices, int slice_first, int slice_count, long long slice_stride_units,
     int* order_log, long long ticks, int* expired) {
@@ -204,9 +224,9 @@ __global__ void __launch_bounds__(64 * kWavesPerBlock) wait_consume_kernel(
             __builtin_amdgcn_s_barrier();   // the three other wavefronts slept here
             const long long part = tile_units * need / nslices;
             for (int k = 0; k < slice_count; ++k)
-                team_copy<true, 64 * kWavesPerBlock, STREAM>(src + glo + (slice_first + k) * part,
-                                                             dst + k * slice_stride_units + glo / nslices, part, mem, tm,
-                                                             (int)threadIdx.x);
+                team_copy_coherent<64 * kWavesPerBlock, STREAM>(src + glo + (slice_first + k) * part,
+                                                                dst + k * slice_stride_units + glo / nslices,
+                                                                (unsigned)part, (unsigned)mem, (unsigned)tm, threadIdx.x);
         }
         lo_base += __shfl(su, 63, 64);
         start_base = (int)(((long long)start_base + __shfl(st, 63, 64)) % members);
@@ -229,7 +249,7 @@ __global__ void __launch_bounds__(kCopyThreads) consume_kernel(const uint4* __re
         else
             count_expired(expired);
     }
-    team_copy<false, kCopyThreads, STREAM>(src + blockIdx.y * units, dst + blockIdx.y * dst_stride_units, units,
+    team_copy<kCopyThreads, STREAM>(src + blockIdx.y * units, dst + blockIdx.y * dst_stride_units, units,
                                            blockIdx.x, gridDim.x, threadIdx.x);
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];   // one slice only
 }

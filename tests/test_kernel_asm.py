@@ -103,8 +103,45 @@ def test_register_budget_and_no_spills(gemm_asm):
     for name, m in meta.items():
         assert m["spill"] == 0, f"{name} spills {m['spill']} registers"
         # 512 registers per SIMD lane: what the GEMM leaves free is all the consumer's wavefronts
-        # (fewer than 64 registers each) have while they run beside it
-        assert m["vgpr"] <= 448, f"{name} takes {m['vgpr']} of 512 registers"
+        # (at most 72 registers each) have while they run beside it
+        assert m["vgpr"] <= 440, f"{name} takes {m['vgpr']} of 512 registers"
+
+
+def _vregs(operand):
+    m = re.fullmatch(r"v\[(\d+):(\d+)\]", operand)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.fullmatch(r"v(\d+)", operand)
+    return {int(m.group(1))} if m else set()
+
+
+def test_no_vector_write_to_the_data_of_a_store_just_issued(gemm_asm):
+    """A store of more than 8 bytes reads its data registers for a cycle or two after issue; a vector
+    instruction that writes one of them right behind it is a hazard.  The compiler keeps its own
+    instructions apart, but the accumulator reads are assembly statements it cannot see into, and it
+    may give them the registers of a store just issued (in an experimental kernel that drained
+    accumulators between stores this corrupted single rows now and then)."""
+    bodies, _ = _kernels(gemm_asm)
+    stores = 0
+    for name, ins in bodies.items():
+        for at, code in enumerate(ins):
+            if not re.match(r"(buffer|global)_store_dwordx[34]", code):
+                continue
+            stores += 1
+            ops = [o.strip().rstrip(",") for o in code.split()[1:]]
+            data = _vregs(ops[0]) if code.startswith("buffer") else _vregs(ops[1])
+            waited = 0
+            for nxt in ins[at + 1:at + 3]:
+                if waited >= 1:
+                    break
+                m = re.match(r"s_nop (\d+)", nxt)
+                if m:
+                    waited += int(m.group(1)) + 1
+                    continue
+                if nxt.startswith("v_"):
+                    assert not (_vregs(nxt.split()[1].rstrip(",")) & data), f"{name}: '{nxt}' right behind '{code}'"
+                waited += 1
+    assert stores > 0
 
 
 def test_consumer_copy_variants_differ_in_their_stores(tmp_path):
@@ -127,8 +164,15 @@ def test_consumer_copy_variants_differ_in_their_stores(tmp_path):
             continue
         if name and line.startswith(".Lfunc_end"):
             name = None
-        if name and "global_store_dwordx4" in line:
+        if name and ("global_store_dwordx4" in line or "buffer_store_dwordx4" in line):
             stores[name][1 if re.search(r"\bnt\b", line.split(";")[0]) else 2] += 1
     assert len(stores) == 4
     for name, (stream, nt, plain) in stores.items():
         assert (nt > 0 and plain == 0) if stream else (plain > 0 and nt == 0), (name, nt, plain)
+    # The persistent consumer's wavefronts share SIMDs with the GEMM's, which take up to 440 of the 512
+    # registers: with more than 72 a resident consumer would keep the GEMM's workgroups from being placed.
+    text = out.read_text()
+    found = re.findall(r"\.name:\s+(_ZN2fo\d+wait_consume_kernel\S+)\n(?:.*\n)*?\s+\.vgpr_count:\s+(\d+)\n\s+\.vgpr_spill_count:\s+(\d+)", text)
+    assert len(found) == 2
+    for name, vgpr, spill in found:
+        assert int(vgpr) <= 72 and int(spill) == 0, (name, vgpr, spill)

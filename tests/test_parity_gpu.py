@@ -729,7 +729,14 @@ def _full_path(L, dev, comm_stream, dt, M, N, K, w, eps, ws=1, a_std=None, b_std
     assert _timeouts(L) == 0
     assert p.dMM.cpu().sum() == 0
     if ws == 1:
-        assert torch.equal(dst, p.dC)                      # staging is the permuted C, bit for bit
+        if not torch.equal(dst, p.dC):                     # staging is the permuted C, bit for bit
+            bad = (dst != p.dC).view(T, BM * BN)
+            slots = bad.any(1).nonzero().flatten().tolist()
+            first = bad[slots[0]].view(BM, BN)
+            raise AssertionError(
+                "staging differs from C in %d slots (first %s): rows %s of slot %d, %d of its bad elements are 0 in staging"
+                % (len(slots), slots[:12], first.any(1).nonzero().flatten().tolist()[:16], slots[0],
+                   int((dst.view(T, BM * BN)[slots[0]][bad[slots[0]]] == 0).sum())))
         out = p.reorder_rmsnorm(dst, eps)
         torch.cuda.synchronize()
         rows = torch.arange(M) if check_rows is None else check_rows
