@@ -59,10 +59,10 @@ PEAK_MFMA_TFLOPS = 2516.6   # MI355X dense fp16/bf16: 256 CU x 4096 FLOP/clk x 2
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 MALL_BYTES = 256 << 20      # memory-side cache: a buffer rotation has to exceed it to measure HBM
 # Bytes that cross the L2 -> memory interface per signalling-GEMM launch, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs of `bench.py --no-overlap` (profiles/gemm_signal_c3_counters.txt):
-# FETCH_SIZE KiB x 1.999 (the 64 MiB consumer copy reads as 32786.5 KiB) + WRITE_SIZE KiB x 1.000.
-# None for workloads that have not been measured.
-MEASURED_TRAFFIC_BYTES = {"c3": 771_800_000}
+# FETCH_SIZE / WRITE_SIZE runs of `bench.py --workload <wl> --no-overlap` (profiles/gemm_traffic_c2_c3_c4_c5.txt):
+# FETCH_SIZE KiB x 2.000 (a 256 MiB consumer copy reads as 131094 KiB) + WRITE_SIZE KiB x 1.000.
+# A workload without a tracked measurement has no entry, and its bench line then has no roofline.traffic.
+MEASURED_TRAFFIC_BYTES = {"c2": 235_200_000, "c3": 772_100_000, "c4": 671_900_000, "c5": 841_500_000}
 
 
 class Timer:
