@@ -15,14 +15,25 @@ import os
 REQUIRED_AFTER_SEARCH = ("BM", "BN", "dur", "Algo", "hint", "cSeg", "rLDN")
 
 
-def gpu_tag(device_name: str) -> str:
+def gpu_tag(device_name: str, arch: str = "") -> str:
     """The reference cuts characters 7..10 out of the device name
-    (tune/search.py:72); on this platform the architecture name is used."""
+    (tune/search.py:72).  Here a product name that is recognised gives its tag;
+    a driver that reports only a generic name ("AMD Radeon Graphics") gives the
+    architecture instead ("gfx950" out of "gfx950:sramecc+:xnack-")."""
     name = device_name.lower()
     for tag in ("mi355x", "mi350x", "mi325x", "mi300x"):
         if tag in name:
             return tag
+    if arch:
+        return arch.split(":")[0].lower()
     return name.replace(" ", "")[-6:] or "gpu"
+
+
+def current_gpu_tag(device: int = 0) -> str:
+    """gpu_tag of a visible device."""
+    import torch
+    props = torch.cuda.get_device_properties(device)
+    return gpu_tag(props.name, getattr(props, "gcnArchName", ""))
 
 
 def config_path(M: int, N: int, K: int, gpu: str, root: str = "configs") -> str:

@@ -262,7 +262,7 @@ def main(argv=None) -> int:
     load()
     dtype = getattr(torch, a.dtype)
     m, n, k = a.m_dim, a.n_dim, a.k_dim
-    gpu = config.gpu_tag(torch.cuda.get_device_properties(0).name)
+    gpu = config.current_gpu_tag()
     path = config.config_path(m, n, k, gpu, a.configs)
     kw = {"warm_up": a.warm_up, "rep": a.rep}
     if os.path.exists(path):

@@ -4,8 +4,9 @@
 What is here: the monitor-mode sampling pass and its majority vote
 (tune/search.py:164-263), the pipeline latency model and the predictive search
 over wave compositions (tune/search.py:316-344, 462-471, 502-513), with the
-consumer copy in the place of the collective.  What is not: the bandwidth-curve
-measurement and the exhaustive timed search, which need real collectives.
+consumer copy in the place of the collective.  The measuring steps around them
+(GEMM profile, bandwidth curve, timed and predictive search, the tuning file)
+are in tune.py.
 
 The vote exists in the reference because its GEMM scheduler is opaque; this
 library's issue order is a known function (tiling.raster_hint), so the sampled

@@ -106,3 +106,89 @@ def test_config_files_use_the_reference_layout(tmp_path):
     with pytest.raises(ValueError, match="hint"):
         config.load_config(path, 4096, 4096)
     assert config.gpu_tag("AMD Instinct MI355X") == "mi355x"
+    assert config.gpu_tag("AMD Radeon Graphics", "gfx950:sramecc+:xnack-") == "gfx950"
+    assert config.gpu_tag("AMD Instinct MI355X", "gfx950:sramecc+:xnack-") == "mi355x"
+
+
+# ---- the tuning driver's host logic (flashoverlap_amd/tune.py)
+
+def test_curve_sizes_follow_the_reference_grid():
+    from flashoverlap_amd import tune
+    sizes = tune.curve_sizes()
+    assert len(sizes) == 36 and sizes[0] == 1 << 20 and sizes[4] == 1 << 21 and sizes[32] == 1 << 28
+    assert all(s % 1024 == 0 for s in sizes) and all(b > a for a, b in zip(sizes, sizes[1:]))
+    assert sizes[1] == int(2 ** 20.25) // 1024 * 1024
+
+
+def test_interpolated_latency_known_answers():
+    from flashoverlap_amd import tune
+    gib = 1024 ** 3
+    curve = [(1 << 20, 100.0), (1 << 22, 300.0), (1 << 24, 300.0)]
+    # on a point: bytes / bandwidth
+    assert tune.interpolate_latency(curve, 1 << 20) == pytest.approx((1 << 21) / (100.0 * gib) * 1000)
+    # half way between two points the bandwidth is their mean
+    mid = ((1 << 20) + (1 << 22)) / 2
+    assert tune.interpolate_latency(curve, mid) == pytest.approx(mid * 2 / (200.0 * gib) * 1000)
+    # outside the curve the end values hold, so the time grows with the size
+    assert tune.interpolate_latency(curve, 1 << 26) == pytest.approx((1 << 27) / (300.0 * gib) * 1000)
+    assert tune.interpolate_latency(curve, 1 << 10) == pytest.approx((1 << 11) / (100.0 * gib) * 1000)
+    # four-byte elements move twice the bytes
+    assert tune.interpolate_latency(curve, 1 << 22, 4) == pytest.approx(2 * tune.interpolate_latency(curve, 1 << 22))
+    for bad in ([], [(1, 2, 3)], [(2, 1.0), (1, 1.0)], [(1, 0.0), (2, 1.0)]):
+        with pytest.raises(ValueError):
+            tune.interpolate_latency(bad, 10)
+
+
+def test_wave_tiles_and_candidates():
+    from flashoverlap_amd import tune
+    assert tune.wave_tiles(128, 128) == 1024 and tune.wave_tiles(256, 128) == 512 and tune.wave_tiles(256, 256, 304) == 304
+    with pytest.raises(ValueError):
+        tune.wave_tiles(96, 128)
+    # c4: 8192 tiles of 128x128 are eight waves
+    all_of_c4 = tune.candidate_csegs(8192, 1024)
+    assert len(all_of_c4) == 2 ** 7 and all(sum(c) == 8192 for c in all_of_c4)
+    assert all_of_c4[0] == [1024] * 8 and all_of_c4[-1] == [8192]
+    assert len({tuple(c) for c in all_of_c4}) == len(all_of_c4)
+    # a last wave that is not full is clipped, never dropped
+    ragged = tune.candidate_csegs(2500, 1024)
+    assert sorted(map(tuple, ragged)) == sorted([(1024, 1024, 452), (1024, 1476), (2048, 452), (2500,)])
+    # groups of two waves at least: four units
+    coarse = tune.candidate_csegs(8192, 1024, 2)
+    assert len(coarse) == 2 ** 3 and all(g % 2048 == 0 for c in coarse for g in c)
+    # the predictive search's pruning: more than five groups only with a first group of one or two units
+    pruned = tune.candidate_csegs(8192, 1024, prune=True)
+    dropped = [c for c in all_of_c4 if c not in pruned]
+    assert dropped and all(len(c) > 5 and c[0] > 2048 for c in dropped)
+    assert all(not (len(c) > 5 and c[0] > 2048) for c in pruned)
+
+
+def test_model_ranking_orders_by_the_pipeline_model():
+    from flashoverlap_amd import tune
+    cands = tune.candidate_csegs(4096, 1024)
+    tile_elems = 128 * 128
+    # a transfer that costs next to nothing: every partition predicts the GEMM time, the order of enumeration stays
+    fast = [(1 << 20, 1e9), (1 << 28, 1e9)]
+    ranked = tune.rank_by_model(1.0, fast, cands, 1024, 4096, tile_elems)
+    assert [c for _, c in ranked][0] == cands[0] and all(t == pytest.approx(1.0, abs=1e-3) for t, _ in ranked)
+    # a slow link (1 GiB/s: the 32 MiB of a wave take 31 ms against 0.25 ms of compute): every prediction
+    # must equal the oracle's recurrence, best first
+    slow = [(1 << 20, 1.0), (1 << 28, 1.0)]
+    ranked = tune.rank_by_model(1.0, slow, cands, 1024, 4096, tile_elems)
+    comm = lambda nbytes: tune.interpolate_latency(slow, nbytes / 2)
+    for t, c in ranked:
+        assert t == pytest.approx(O.predict_latency_literal(1.0, comm, c, 1024, 4096, tile_elems * 2))
+    assert [t for t, _ in ranked] == sorted(t for t, _ in ranked)
+    assert ranked[-1][1] == [4096]          # nothing overlapped is the worst when the link is the bottleneck
+
+
+def test_profile_lists_are_read_back(tmp_path):
+    from flashoverlap_amd import tune
+    path = str(tmp_path / "m1n1k1_x.json")
+    config.save_profile(path, [128, 256], [128, 128], [0.2, 0.3], [1, 5])
+    assert tune.load_profile(path) == ([128, 256], [128, 128], [0.2, 0.3], [1, 5])
+    config.save_solution(path, 128, 128, 0.2, 1, [0], [1])
+    assert tune.load_profile(path) == ([128], [128], [0.2], [1])
+    json.dump({"BM": [128]}, open(path, "w"))
+    with pytest.raises(ValueError, match="profile step"):
+        tune.load_profile(path)
+    assert tune.curve_path("all_reduce", 1, "cfg").endswith("cfg/bandwidth_all_reduce_tp1.pt")
