@@ -546,10 +546,13 @@ int choose_macro_tile(int BM, int BN, int M, int N, bool any_shape) {
     // that is an odd multiple of 128 is covered by half a macro tile.  The plain GEMM has no
     // layout to respect: any M and N, either macro tile.
     const bool ok128 = any_shape || (BM == 128 && BN == 128);
+    if (const int forced = knob(knobs().macro_tile); forced == 256 || (forced == 128 && ok128)) return forced;   // fo_tune
     if (ok128) {
-        // Small problems: prefer the tile that puts work on more CUs.
+        // Problems of up to half a round of 256x256 tiles: the 128x128 macro tile, of which a CU
+        // holds two workgroups, keeps all CUs busy in one round (fp16, K = 4096: 2048x4096 64 us
+        // against 80, level with the vendor library; from 160 macro tiles on the large tile wins).
         const int wg256 = ((M + 255) / 256) * ((N + 255) / 256);
-        if (wg256 < 128) return 128;
+        if (wg256 <= 128) return 128;
     }
     return 256;
 }

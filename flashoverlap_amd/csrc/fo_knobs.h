@@ -13,6 +13,7 @@ struct Knobs {
     std::atomic<int> release_mode{1};           // 1 = write-through tile stores, acknowledged, then a relaxed atomic; 0 = release-ordered atomic
     std::atomic<int> copy_streaming_stores{2};  // consumer copies: 0 ordinary stores, 1 non-temporal, 2 chosen per launch
     std::atomic<int> wait_timeout_ms{10000};    // bound of every device-side wait
+    std::atomic<int> macro_tile{0};             // 0 = chosen per shape, 128 or 256 = forced where the layout tile allows it
 };
 
 inline Knobs& knobs() {
@@ -29,6 +30,8 @@ inline bool set_knob(std::string_view key, int value) {
     else if (key == "release_mode") k.release_mode.store(value ? 1 : 0, std::memory_order_relaxed);
     else if (key == "copy_streaming_stores" && value >= 0 && value <= 2)
         k.copy_streaming_stores.store(value, std::memory_order_relaxed);
+    else if (key == "macro_tile" && (value == 0 || value == 128 || value == 256))
+        k.macro_tile.store(value, std::memory_order_relaxed);
     else return false;
     return true;
 }

@@ -158,7 +158,12 @@ int fo_raster_hint(int algo, int M, int N, int* hint_host);
  *                  memory-side cache), ordinary stores in smaller ones and in
  *                  fo_settle_consume (their destination is then still cached
  *                  for the kernel that reads it next); 1: non-temporal
- *                  everywhere; 0: ordinary everywhere. */
+ *                  everywhere; 0: ordinary everywhere.
+ *   "macro_tile"   the tile one workgroup computes.  0 (default): chosen per
+ *                  shape (128x128 for outputs of up to 128 tiles of 256x256,
+ *                  else 256x256); 128 or 256: forced, 128 only where the
+ *                  layout tile is 128x128 or the GEMM is the plain one.  The
+ *                  issue order fo_raster_hint reports follows the setting. */
 int fo_tune(const char* key, int value);
 
 /* ---- counting / wait -------------------------------------------------- */

@@ -106,3 +106,48 @@ def test_reorder_rmsnorm_long_rows(L, dev, dt, bs, dim, BM, BN, rldn):
     assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and O.max_abs(out.cpu(), ref) < MAX_ABS_TOL
     ulp = 2 ** -10 if dt == torch.float16 else 2 ** -7
     assert ((out.cpu().float() - ref.float()).abs() <= 2 * ulp * ref.float().abs() + 1e-6).all()
+
+
+def test_macro_tile_knob_changes_the_schedule_not_the_result(L, dev):
+    """fo_tune "macro_tile": either workgroup tile gives the same bits, the issue order follows the
+    setting, and a value the knob does not take is refused."""
+    M, N, K = 2048, 4096, 264            # 128 tiles of 256x256: the shape at which the automatic choice changes over
+    g = torch.Generator().manual_seed(5)
+    A = torch.randint(-2, 3, (M, K), generator=g).to(torch.bfloat16)
+    B = torch.randint(-2, 3, (N, K), generator=g).to(torch.bfloat16)
+    dA, dB = A.to(dev), B.to(dev)
+    want = O.gemm(A, B)
+    hints = {}
+    order_of_256x128 = capi.raster_hint(4, M, N)
+    try:
+        for mt in (128, 256, 0):
+            capi.check(L.fo_tune(b"macro_tile", mt))
+            D = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=dev)
+            capi.check(L.fo_gemm(capi.FO_BF16, 1, M, N, K, dA.data_ptr(), dB.data_ptr(), D.data_ptr(), None))
+            torch.cuda.synchronize()
+            assert torch.equal(D.cpu(), want), mt
+            hints[mt] = capi.raster_hint(1, M, N)
+            assert sorted(hints[mt]) == list(range((M // 128) * (N // 128)))
+            # a signalling launch under the same setting: counters full, placement by RA
+            T = (M // 128) * (N // 128)
+            ra = torch.tensor(hints[mt], dtype=torch.int64)
+            RA = torch.empty(T, dtype=torch.int32)
+            RA[ra] = torch.arange(T, dtype=torch.int32)
+            cseg = torch.tensor([T // 2, T - T // 2], dtype=torch.int32, device=dev)
+            MM = torch.zeros(64, dtype=torch.int32, device=dev)
+            dRA = RA.to(dev)
+            capi.check(L.fo_gemm_signal(capi.FO_BF16, 1, M, N, K, 1, cseg.data_ptr(), 2, None, dA.data_ptr(), dB.data_ptr(),
+                                        D.data_ptr(), MM.data_ptr(), dRA.data_ptr(), 0, None))
+            torch.cuda.synchronize()
+            assert MM[:2].cpu().tolist() == [T // 2, T - T // 2]
+            assert torch.equal(D.cpu().reshape(-1), O.place_tiles(want, RA.numpy().reshape(M // 128, N // 128), 128, 128, 1).reshape(-1))
+        assert hints[128] != hints[256] and hints[0] == hints[128]      # up to 128 large tiles: the small one
+        # the first workgroup of the large tile covers four layout tiles, that of the small tile one
+        assert sorted(hints[256][:4]) == [0, 1, N // 128, N // 128 + 1] and hints[128][0] == 0
+        assert L.fo_tune(b"macro_tile", 64) != 0
+        # a 256x128 layout tile cannot be served by the small workgroup tile: the setting is ignored there
+        capi.check(L.fo_tune(b"macro_tile", 128))
+        assert capi.raster_hint(4, M, N) == order_of_256x128
+    finally:
+        capi.check(L.fo_tune(b"macro_tile", 0))
+

@@ -58,3 +58,20 @@ def test_speed_table_on_config1(dev, comm_op, ws):
         torch.cuda.synchronize()
         assert O.rel_l2(D.cpu(), cref[: M // ws]) < 1e-3
     assert O.rel_l2(C.cpu(), cref) < 1e-3
+
+
+def test_gemm_sweep_table(dev):
+    """test/sweep_gemm.py on two shapes, one of them no multiple of any tile: every row has a vendor time, the
+    best Algo's time and their ratio; a shape the GEMM refuses is reported as failed, as the reference does,
+    and left out of the summary."""
+    from flashoverlap_amd import sweep_gemm
+    lines = []
+    results = sweep_gemm.sweep([1024, 1000], [1024], [512], torch.float16, out=lines.append, warm_up=2, rep=5)
+    assert lines[0] == sweep_gemm.HEADER
+    assert len(results) == 2 and [r[:3] for r in results] == [(1024, 1024, 512), (1000, 1024, 512)]
+    for M, N, K, algo, vendor, ours, ratio in results:
+        assert 0 <= algo < capi.lib().fo_algo_count() and vendor > 0 and ours > 0 and ratio == pytest.approx(ours / vendor)
+    assert any("--- Top 10 closest" in l for l in lines)
+    lines = []
+    assert sweep_gemm.sweep([1024], [1024], [500], torch.float16, out=lines.append, warm_up=1, rep=2) == []
+    assert "FAIL" in lines[2] and not any("--- Top 10" in l for l in lines)

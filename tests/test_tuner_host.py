@@ -192,3 +192,14 @@ def test_profile_lists_are_read_back(tmp_path):
     with pytest.raises(ValueError, match="profile step"):
         tune.load_profile(path)
     assert tune.curve_path("all_reduce", 1, "cfg").endswith("cfg/bandwidth_all_reduce_tp1.pt")
+
+
+def test_sweep_rows_follow_the_reference_table():
+    from flashoverlap_amd import sweep_gemm
+    assert sweep_gemm.note_for(1.0) == "<== CLOSE" and sweep_gemm.note_for(1.1) == "<== CLOSE"
+    assert sweep_gemm.note_for(1.2) == "<= OK" and sweep_gemm.note_for(1.3) == "<= OK" and sweep_gemm.note_for(1.31) == ""
+    row = sweep_gemm.format_row(1024, 2048, 4096, 3, 0.5, 0.6)
+    assert row.split() == ["1024", "2048", "4096", "3", "0.5000", "0.6000", "1.20", "<=", "OK"]
+    assert len(row) == len(sweep_gemm.HEADER)
+    failed = sweep_gemm.format_row(1024, 2048, 4096, -1, 0.5, None)
+    assert failed.split() == ["1024", "2048", "4096", "FAIL", "0.5000", "N/A", "N/A"]
