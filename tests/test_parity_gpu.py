@@ -406,6 +406,7 @@ def test_scatter_epilogue_and_reducescatter_slices(L, dev, comm_stream, ws, cseg
     assert p.dMM.cpu()[:p.G].tolist() == cseg
     # consumer: all ws receive buffers side by side
     D = torch.zeros(ws, M * N // ws, dtype=p.dt, device=dev)
+    torch.cuda.synchronize()         # the second stream is not ordered behind torch's: D must be cleared before it is written
     capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), D.data_ptr(), BM * BN,
                                  ws, 0, ws, M * N // ws, None, 4, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
@@ -420,8 +421,9 @@ def test_scatter_epilogue_and_reducescatter_slices(L, dev, comm_stream, ws, cseg
         ref = O.rmsnorm(natural[k::ws], p.gamma, 1e-5)
         assert O.rel_l2(out.cpu(), ref) < REL_L2_TOL and _max_abs_ok(out.cpu(), ref)
     # one rank's view: only slice 1
-    p.gemm_signal()
     one = torch.zeros(M * N // ws, dtype=p.dt, device=dev)
+    torch.cuda.synchronize()
+    p.gemm_signal()
     capi.check(L.fo_wait_consume(p.dcseg.data_ptr(), p.G, p.dMM.data_ptr(), p.dC.data_ptr(), one.data_ptr(), BM * BN,
                                  ws, 1, 1, 0, None, 2, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
@@ -552,6 +554,7 @@ def test_wait_kernel_resets_counter_and_is_bounded(L, dev, comm_stream):
         dst = torch.zeros_like(src)
         bad = torch.tensor([1, 1], dtype=torch.int32, device=dev)
         flags = torch.tensor([1, 0], dtype=torch.int32, device=dev)   # group 1 never completes
+        torch.cuda.synchronize()     # src and dst are filled on torch's stream, the consumer runs on another
         capi.check(L.fo_wait_consume(bad.data_ptr(), 2, flags.data_ptr(), src.data_ptr(), dst.data_ptr(), 2048, 1, 0,
                                      1, 0, None, 3, None, comm_stream))
         capi.check(L.fo_stream_sync(comm_stream))
@@ -569,11 +572,13 @@ def test_settle_consume_clears_the_right_count_and_reports_a_wrong_one(L, dev, c
     mm = torch.tensor([7, 9, 0], dtype=torch.int32, device=dev)
     src = torch.randint(-30000, 30000, (40000,), dtype=torch.int16, device=dev)
     dst = torch.zeros_like(src)
+    torch.cuda.synchronize()         # filled on torch's stream, copied on another that is not ordered behind it
     capi.check(L.fo_settle_consume(7, mm.data_ptr(), src.data_ptr(), dst.data_ptr(), 2 * 40000, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 0 and torch.equal(dst, src)
     # a wrong count stays where it is and is counted, at once (no polling); the copy is still made
     dst.zero_()
+    torch.cuda.synchronize()
     capi.check(L.fo_settle_consume(8, mm.data_ptr() + 4, src.data_ptr(), dst.data_ptr(), 2 * 40000, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
     assert mm.cpu().tolist() == [0, 9, 0] and _timeouts(L) == 1 and torch.equal(dst, src)
@@ -591,6 +596,7 @@ def test_consume_slices_equals_one_copy_per_slice(L, dev, comm_stream):
     src = torch.randint(-30000, 30000, (ws * part + 64,), dtype=torch.int16, device=dev)
     want = torch.full((ws * stride,), -1, dtype=torch.int16, device=dev)
     got = want.clone()
+    torch.cuda.synchronize()         # filled on torch's stream, copied on another that is not ordered behind it
     for k in range(ws):
         capi.check(L.fo_consume(src.data_ptr() + 2 * (64 + k * part), want.data_ptr() + 2 * k * stride, 2 * part,
                                 comm_stream))
@@ -602,6 +608,7 @@ def test_consume_slices_equals_one_copy_per_slice(L, dev, comm_stream):
     # with a counter: settled once, by the launch as a whole
     mm = torch.tensor([5], dtype=torch.int32, device=dev)
     got.fill_(-1)
+    torch.cuda.synchronize()
     capi.check(L.fo_consume_slices(5, mm.data_ptr(), src.data_ptr() + 2 * 64, got.data_ptr(), 2 * part, ws, 2 * stride,
                                    capi.FO_COPY_CACHED, None, comm_stream))
     capi.check(L.fo_stream_sync(comm_stream))
