@@ -25,6 +25,7 @@ from __future__ import annotations
 import argparse
 import os
 import sys
+import time
 
 import torch
 
@@ -35,10 +36,23 @@ REP = 200
 TILES_PER_WAVE_256 = 256   # workgroups resident at a time: one 256x256 macro tile per CU
 
 
+WARM_UP_MS = 60.0   # the warm-up also lasts at least this long
+
+
 def _timed(fn, warm_up=WARM_UP, rep=REP):
-    """Mean milliseconds of fn() over `rep` iterations, one event pair each (test/test.py:157-164)."""
+    """Mean milliseconds of fn() over `rep` iterations, one event pair each (test/test.py:157-164).
+    The warm-up is the reference's 20 iterations and, beyond it, as many more as it takes to keep
+    the GPU busy for WARM_UP_MS: a column measured right after a light one (the GEMM rows after the
+    copy row) otherwise starts on a chip that has clocked down and reads 2-3 % slow."""
     for _ in range(warm_up):
         fn()
+    if warm_up >= WARM_UP:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1000.0 < WARM_UP_MS:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
     start = [torch.cuda.Event(enable_timing=True) for _ in range(rep)]
     end = [torch.cuda.Event(enable_timing=True) for _ in range(rep)]
     for i in range(rep):
@@ -133,7 +147,6 @@ def perf_running(M, N, K, BM, BN, Algo, cSeg, hint, comm_op, world_size=1, dtype
     dur = _timed(fn, **kw)
     if keep is not None:
         # host time to enqueue one call (nothing is waited for): what the torch-API path costs the CPU
-        import time
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(20):
