@@ -313,10 +313,11 @@ def main() -> int:
     # milliseconds of load then run 3-6 % slow, which with a short --steps/--warmup is all that would
     # be measured.  Steps are therefore run, untimed, until the chip has been busy for --settle-ms;
     # the W warm-up steps and the K timed steps of every pass follow as the contract says.
-    settled_ms, t_settle = 0.0, time.perf_counter()
+    settled_ms, settle_steps, t_settle = 0.0, 0, time.perf_counter()
     while a.settle_ms > 0 and settled_ms < a.settle_ms:
         for _ in range(20):
             step(grp, not a.no_overlap)
+        settle_steps += 20
         torch.cuda.synchronize()
         settled_ms = (time.perf_counter() - t_settle) * 1e3
     # the timed steps, then the same steps again with the kernels' event pairs attached
@@ -465,7 +466,7 @@ def main() -> int:
         "value_is": "2*M*N*K / whole step time (signalling GEMM || consumer, then reorder+RMSNorm); "
                     "the signalling GEMM kernel's own rate is gemm_kernel_tflops = roofline.achieved",
         "gemm_kernel_tflops": round(flops / step_gemm_ms / 1e9, 2),
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "clock_settle_ms": round(settled_ms, 1),
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "clock_settle_ms": round(settled_ms, 1), "clock_settle_steps": settle_steps,
         "ms_per_step": round(step_ms, 5),
         "ms_per_step_with_kernel_events": round(step_probed_ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dts, "data": "synthetic",
