@@ -36,6 +36,28 @@ def current_gpu_tag(device: int = 0) -> str:
     return gpu_tag(props.name, getattr(props, "gcnArchName", ""))
 
 
+def current_gpu_tags(device: int = 0) -> list:
+    """Tags under which a tuning file of the visible device may have been saved: the product tag
+    if the driver reports one, then the architecture (the same silicon reports either, depending
+    on the driver)."""
+    import torch
+    props = torch.cuda.get_device_properties(device)
+    arch = getattr(props, "gcnArchName", "").split(":")[0].lower()
+    tags = [gpu_tag(props.name, arch)]
+    if arch and arch not in tags:
+        tags.append(arch)
+    return tags
+
+
+def find_config(M: int, N: int, K: int, tags, root: str = "configs") -> str:
+    """Path of the first existing tuning file among the tags, else the path under the first tag."""
+    for tag in tags:
+        path = config_path(M, N, K, tag, root)
+        if os.path.exists(path):
+            return path
+    return config_path(M, N, K, tags[0], root)
+
+
 def config_path(M: int, N: int, K: int, gpu: str, root: str = "configs") -> str:
     return os.path.join(root, f"m{M}n{N}k{K}_{gpu}.json")
 

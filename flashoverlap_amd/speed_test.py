@@ -275,8 +275,7 @@ def main(argv=None) -> int:
     load()
     dtype = getattr(torch, a.dtype)
     m, n, k = a.m_dim, a.n_dim, a.k_dim
-    gpu = config.current_gpu_tag()
-    path = config.config_path(m, n, k, gpu, a.configs)
+    path = config.find_config(m, n, k, config.current_gpu_tags(), a.configs)
     kw = {"warm_up": a.warm_up, "rep": a.rep}
     if os.path.exists(path):
         cfg = config.load_config(path, m, n)

@@ -108,6 +108,10 @@ def test_config_files_use_the_reference_layout(tmp_path):
     assert config.gpu_tag("AMD Instinct MI355X") == "mi355x"
     assert config.gpu_tag("AMD Radeon Graphics", "gfx950:sramecc+:xnack-") == "gfx950"
     assert config.gpu_tag("AMD Instinct MI355X", "gfx950:sramecc+:xnack-") == "mi355x"
+    # a file saved under the architecture is found by a driver that reports the product, and the other way round
+    config.save_profile(config.config_path(8, 8, 8, "gfx950", str(tmp_path)), [128], [128], [0.1], [1])
+    assert config.find_config(8, 8, 8, ["mi355x", "gfx950"], str(tmp_path)).endswith("m8n8k8_gfx950.json")
+    assert config.find_config(8, 8, 16, ["mi355x", "gfx950"], str(tmp_path)).endswith("m8n8k16_mi355x.json")
 
 
 # ---- the tuning driver's host logic (flashoverlap_amd/tune.py)
