@@ -151,3 +151,48 @@ def test_macro_tile_knob_changes_the_schedule_not_the_result(L, dev):
     finally:
         capi.check(L.fo_tune(b"macro_tile", 0))
 
+
+
+@pytest.mark.parametrize("M,N,K", [(8191, 4097, 7168), (8190, 4088, 7160)])
+def test_plain_gemm_ragged_at_full_size(L, dev, M, N, K):
+    """The c3 shape with one row and column missing / one added (N odd: element-wise stores; N a multiple of 8:
+    16-byte stores with a ragged last tile): sampled rows against the oracle, and, for the whole output, two
+    properties that hold at any size — integer-valued operands give the exact product, which is linear in A."""
+    dt = torch.bfloat16
+    print(f"ragged full size {M}x{N}x{K}", flush=True)
+    g = torch.Generator().manual_seed(M + N)
+    A = (torch.randn(M, K, generator=g)).to(dt)
+    B = (0.02 * torch.randn(N, K, generator=g)).to(dt)
+    dA, dB = A.to(dev), B.to(dev)
+    buf = torch.full((GUARD + M * N + 8 + GUARD,), 7.0, dtype=dt, device=dev)
+    start = GUARD + (-(buf.data_ptr() // 2 + GUARD) % 8)           # 16-byte aligned output
+    D = buf[start:start + M * N]
+    assert D.data_ptr() % 16 == 0
+    capi.check(L.fo_gemm(capi.FO_BF16, 1, M, N, K, dA.data_ptr(), dB.data_ptr(), D.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert (buf[:start] == 7.0).all() and (buf[start + M * N:] == 7.0).all()
+    rows = torch.tensor([0, 1, 127, 128, 255, 256, 4095, 4096, M - 257, M - 256, M - 2, M - 1])
+    ref = O.gemm_fp32(A[rows], B).to(dt)
+    got = D.view(M, N)[rows.to(dev)].cpu()
+    assert O.rel_l2(got, ref) < REL_L2_TOL and O.max_abs(got, ref) < MAX_ABS_TOL
+    # exact arithmetic: operands in {-1, 0, 1} (products and sums of up to K of them are exact in fp32 and,
+    # for |sum| <= 256, in bf16); D(A1) + D(A2) == D(A1 + A2) where the supports of A1 and A2 do not overlap
+    A1 = torch.zeros(M, K, dtype=dt)
+    A2 = torch.zeros(M, K, dtype=dt)
+    A1[:, 0:200:2] = torch.randint(-1, 2, (M, 100), generator=g).to(dt)
+    A2[:, 1:201:2] = torch.randint(-1, 2, (M, 100), generator=g).to(dt)
+    Bi = torch.zeros(N, K, dtype=dt)
+    Bi[:, :200] = torch.randint(-1, 2, (N, 200), generator=g).to(dt)
+    dBi = Bi.to(dev)
+    outs = []
+    for Ax in (A1, A2, A1 + A2):
+        dAx = Ax.to(dev)
+        Dx = torch.empty(M * N, dtype=dt, device=dev)
+        capi.check(L.fo_gemm(capi.FO_BF16, 1, M, N, K, dAx.data_ptr(), dBi.data_ptr(), Dx.data_ptr(), None))
+        torch.cuda.synchronize()
+        outs.append(Dx.float())
+    assert torch.equal(outs[0] + outs[1], outs[2])
+    assert outs[2].abs().max() <= 200 and outs[2].abs().sum() > 0
+    # and the corner block against the oracle, exactly
+    corner = outs[2].view(M, N)[M - 300:, N - 300:].cpu()
+    assert torch.equal(corner, O.gemm_fp32((A1 + A2)[M - 300:], Bi[N - 300:]))
