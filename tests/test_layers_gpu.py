@@ -120,3 +120,25 @@ def test_monitor_sampling_and_vote_agree_with_the_raster(ready):
     agree = len(set(hint[:wave]) & set(issued[:wave])) / wave
     print("first-wave agreement between sampled and analytic hint: %.3f" % agree, flush=True)
     assert agree > 0.9
+
+
+@pytest.mark.parametrize("comm_op,ws,rank,dt", [("all_reduce", 1, 0, torch.float16), ("reduce_scatter", 8, 3, torch.bfloat16)])
+def test_correctness_examples(ready, tmp_path, comm_op, ws, rank, dt):
+    """The two example scripts of the reference as one command: its verdict lines, and True."""
+    from flashoverlap_amd import correctness
+    M, N, K = 2048, 1024, 512
+    cfg = _config(M, N, 1, 32, tmp_path)
+    said = []
+    assert correctness.run(comm_op, M, N, K, cfg, ws, rank, dt, out=said.append)
+    want = "[GEMM+AllReduce+RMSNorm] all close :  True" if comm_op == "all_reduce" else "[GEMM+ReduceScatter+RMSNorm] all close :  True"
+    assert said[-1] == want
+    if comm_op == "reduce_scatter":
+        assert said[0].startswith("Index of max absolute difference") and len(said) == 5
+    # a cSeg that does not add up to the tiles is refused: by the overlapped call, or already by the row map
+    bad = dict(cfg, cSeg=cfg["cSeg"][:-1])
+    with pytest.raises((RuntimeError, ValueError)):
+        correctness.run(comm_op, M, N, K, bad, ws, rank, dt, out=lambda s: None)
+    # the command line, on a shape without a tuning file
+    assert correctness.main(["--m_dim", "1024", "--n_dim", "1024", "--k_dim", "256", "--comm_op", comm_op,
+                             "--world_size", str(ws), "--rank", str(rank), "--dtype", str(dt).split(".")[1],
+                             "--configs", str(tmp_path)]) == 0
