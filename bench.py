@@ -367,10 +367,21 @@ def main() -> int:
     capi.check(L.fo_tune(b"release_mode", default_release_mode))
     grp.MM.zero_()
     pl_ms, pl_min = time_kernel(lambda i: gemm_plain(), it)
+    # Every buffer of the rotation holds the step's real output: on an all-zero input the kernel runs
+    # 9 % faster than on data (20.4 against 22.5 us on c3), which a rotation over one real and two
+    # cleared buffers used to credit to it.
+    for other_staging in stagings[1:]:
+        other_staging.copy_(stagings[0])
+    torch.cuda.synchronize()
     rms_rot_ms, _ = time_kernel(lambda i: norm(i % npairs), it)      # rotation larger than the memory-side cache
     rms_same_ms, rms_min = time_kernel(lambda i: norm(0), it)         # one pair over and over: served by that cache
     cons_ms, _ = time_kernel(
         lambda i: capi.check(L.fo_consume(Cp.data_ptr(), stagings[i % npairs].data_ptr(), 2 * M * N, main_stream)), it)
+    # the yardstick for reorder+RMSNorm: the copy kernel over the same rotation, source and destination both
+    # rotating (the consumer's copy above reads one source over and over, which the memory-side cache then holds)
+    rot_copy_ms, _ = time_kernel(
+        lambda i: capi.check(L.fo_consume(stagings[i % npairs].data_ptr(), outs[i % npairs].data_ptr(), 2 * M * N,
+                                          main_stream)), it)
     # The same instruction stream on all-zero operands: the MFMAs toggle nothing, the chip stays
     # below its power limit and keeps its clock.  What separates this figure from gemm_plain is
     # the power limit, not the kernel's schedule.
@@ -512,8 +523,9 @@ def main() -> int:
                             "in_step": hbm(step_norm_ms),
                             "same_pair_back_to_back": {**hbm(rms_same_ms), "min_single_launch_us": round(rms_min * 1e3, 2)},
                             # the yardstick of the same run: a plain copy kernel moving the same bytes over the same rotation
-                            "copy_kernel_same_run": {"achieved": round(cons_bytes / cons_ms / 1e6, 1),
-                                                     "frac": round(cons_bytes / cons_ms / 1e6 / PEAK_HBM_GBPS, 4)}},
+                            "copy_kernel_same_run": {"achieved": round(cons_bytes / rot_copy_ms / 1e6, 1),
+                                                     "frac": round(cons_bytes / rot_copy_ms / 1e6 / PEAK_HBM_GBPS, 4),
+                                                     "avg_us": round(rot_copy_ms * 1e3, 2)}},
         "consume_copy": {"achieved": round(cons_bytes / cons_ms / 1e6, 1), "unit": "GB/s",
                          "avg_us": round(cons_ms * 1e3, 2)},
         "other_reading": other,

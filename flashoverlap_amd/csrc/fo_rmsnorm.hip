@@ -41,9 +41,9 @@ constexpr int kWideThreads = 256;  // rows too long for one wavefront's register
 
 // Ordinary loads, streaming (non-temporal) stores: the result is not read again here, and it
 // must not displace the GEMM operands held in the memory-side cache.  Measured on 8192 x 4096
-// against this choice: non-temporal loads 26 us instead of 20 over rotating buffers, ordinary
-// stores 28; the other cache-policy bits on the stores (sc1, sc0 sc1, with and without nt) equal
-// or slower.
+// against this choice (inside a step / one buffer pair back to back, 21.8 / 21.7 us as it is):
+// non-temporal loads 21.8 / 25.5, ordinary stores 23.9 / 22.2; the other cache-policy bits on the
+// stores (sc1, sc0 sc1, with and without nt) equal or slower.
 template <typename V>
 __device__ __forceinline__ V load_row_chunk(const V* p) {
     return *p;
