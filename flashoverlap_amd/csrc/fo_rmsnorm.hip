@@ -1,8 +1,11 @@
 // RMSNorm and reorder+RMSNorm for gfx950: one 64-lane wavefront per output row,
 // the whole row held in registers between the sum of squares and the scaling,
 // 128-bit coalesced HBM accesses, a wavefront butterfly for the reduction (no
-// LDS, no barrier); gamma is fetched together with the row so that nothing but
-// arithmetic sits between the last load and the first store.  (Rows of more
+// LDS in the reduction).  gamma is staged in LDS once per workgroup while the rows' loads
+// are in flight and read from there chunk by chunk behind the reduction: held in registers
+// beside the row it doubled the kernel's footprint (81 registers at dim 4096, 330 at 16384:
+// a single wavefront per SIMD), and the registers decide how many rows a SIMD has in
+// flight.  (Rows of more
 // than 16384 elements take a second kernel: one workgroup per row, two passes.)  The reorder
 // variant gathers the row from the tile-permuted GEMM output: 16 consecutive
 // lanes read one 256-byte row segment of a 128-wide tile, so every access is
@@ -61,22 +64,34 @@ struct NormParams {
     float eps;
 };
 
-// CH = 16-byte chunks per lane (dim <= CH * 512).
+// CH = 16-byte chunks per lane (dim <= CH * 512).  GAMMA_IN_LDS: see the head of the file; measured per CH
+// (reorder / plain, against gamma in registers, same box): CH 2 -3 % / -13 %, CH 4 -4 % / +3 %, CH 8 -1...-7 % /
+// -8 %, CH 32 -37 % / -10 %, but CH 16 +2 % / +4 % on 16384 x 8192 (more rows in flight than that size likes),
+// so CH 16 keeps gamma in registers.
+template <int CH>
+constexpr bool gamma_in_lds() { return CH != 16; }
+
 template <typename T, int CH, int MODE>
 __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __restrict__ x0, const T* __restrict__ gamma,
                                                       T* __restrict__ out0, const int* __restrict__ RA,
                                                       const NormParams p) {
     using vec = typename Vec8<T>::type;
+    constexpr bool GAMMA_IN_LDS = gamma_in_lds<CH>();
+    extern __shared__ __attribute__((aligned(16))) unsigned char norm_smem[];   // dim * 2 bytes when gamma is staged
+    vec* lds_gamma = (vec*)norm_smem;
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
-    if (row >= p.bs) return;
+    const int row_of_wave = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    const bool live = row_of_wave < p.bs;
+    if (!GAMMA_IN_LDS && !live) return;
+    const int row = live ? row_of_wave : p.bs - 1;   // a wavefront beyond the last row stays for the barrier, loading a row it never stores
     // blockIdx.y selects one of several independent [bs, dim] problems laid out back to back
     const T* __restrict__ x = x0 + (size_t)blockIdx.y * p.bs * p.dim;
     T* __restrict__ out = out0 + (size_t)blockIdx.y * p.bs * p.dim;
 
     const int dim = p.dim;
     const int nchunk = dim >> 3;
-    vec xv[CH], gv[CH];
+    vec xv[CH];
+    [[maybe_unused]] vec gv[GAMMA_IN_LDS ? 1 : CH];
     if constexpr (MODE == kNormGatherFast) {
         // tiles of this row: RA[tile_row .. tile_row + ldn), ldn <= 64: one entry per lane
         const int ldn = dim >> p.log_bn;
@@ -116,10 +131,16 @@ __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __
             if (c < nchunk) xv[k] = load_row_chunk((const vec*)(xr + (c << 3)));
         }
     }
+    if constexpr (GAMMA_IN_LDS) {
+        for (int c = threadIdx.x; c < nchunk; c += 64 * kRowsPerBlock) lds_gamma[c] = *(const vec*)(gamma + (c << 3));
+        __syncthreads();
+        if (!live) return;
+    } else {
 #pragma unroll
-    for (int k = 0; k < CH; ++k) {
-        const int c = k * 64 + lane;
-        if (c < nchunk) gv[k] = *(const vec*)(gamma + (c << 3));
+        for (int k = 0; k < CH; ++k) {
+            const int c = k * 64 + lane;
+            if (c < nchunk) gv[k] = *(const vec*)(gamma + (c << 3));
+        }
     }
 
     float ss = 0.f;
@@ -147,11 +168,13 @@ __global__ void __launch_bounds__(64 * kRowsPerBlock) rmsnorm_kernel(const T* __
     for (int k = 0; k < CH; ++k) {
         const int c = k * 64 + lane;
         if (c < nchunk) {
-            vec o;
+            vec o, g;
+            if constexpr (GAMMA_IN_LDS) g = lds_gamma[c];
+            else g = gv[k];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const T y = (T)((float)xv[k][e] * scale);
-                o[e] = (T)((float)y * (float)gv[k][e]);
+                o[e] = (T)((float)y * (float)g[e]);
             }
             store_row_chunk(o, (vec*)(orow + (c << 3)));
         }
@@ -249,11 +272,12 @@ static int launch_t(const void* x, const void* gamma, void* out, const int* RA, 
     const dim3 grid((p.bs + kRowsPerBlock - 1) / kRowsPerBlock, nbatch), block(64 * kRowsPerBlock);
 #define FO_RMS_CASE(CH)                                                                                           \
     do {                                                                                                          \
+        const size_t smem = gamma_in_lds<CH>() ? (size_t)p.dim * sizeof(T) : 0;                                   \
         if (timer.start)                                                                                          \
-            hipExtLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, 0, stream, timer.start, timer.stop, \
-                                  0, (const T*)x, (const T*)gamma, (T*)out, RA, p);                               \
+            hipExtLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, smem, stream, timer.start,          \
+                                  timer.stop, 0, (const T*)x, (const T*)gamma, (T*)out, RA, p);                   \
         else                                                                                                      \
-            hipLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, 0, stream, (const T*)x,                \
+            hipLaunchKernelGGL((rmsnorm_kernel<T, CH, MODE>), grid, block, smem, stream, (const T*)x,             \
                                (const T*)gamma, (T*)out, RA, p);                                                  \
     } while (0)
     if (ch <= 1) FO_RMS_CASE(1);
