@@ -4,7 +4,7 @@
 // MI355X dispatches workgroup i of a grid to XCD i % 8, and every XCD has its
 // own L2.  The unit of the map is a block of kGroupM x 4 macro tiles: the 32
 // workgroups one XCD runs at a time, which share their A and B panels in that
-// L2.  Units are ordered band by band (a band = kGroupM rows of macro tiles,
+// L2 (numbered row by row inside the block).  Units are ordered band by band (a band = kGroupM rows of macro tiles,
 // all columns), and the eight units of one hardware wave (256 workgroups) go to
 // the eight XCDs.  So the XCDs of a wave work on the same A rows, which the
 // memory-side cache then fetches from HBM once for all of them (with each XCD
@@ -47,23 +47,22 @@ FO_HD TileCoord raster_map(int pid, int GM, int GN, unsigned gn_magic) {
     const int whole = total / kWave * kWave;
     const int pos = pid < whole ? ((local / kUnit) * kXcds + xcd) * kUnit + local % kUnit : pid;
     // Position -> tile: bands of kGroupM rows (the last may be lower), in a band blocks of kUnitN
-    // columns (the last may be narrower), in a block column by column.
+    // columns (the last may be narrower), in a block row by row.  (Row by row, not column by
+    // column: the slots of the tiles that one output row crosses are then a few slots apart
+    // inside a block and one block apart between blocks, where column by column they were 256
+    // slots = 8 MiB apart, a stride at which the segments that reorder+RMSNorm gathers for a row
+    // fall into few memory channels: that kernel ran 5-7 % longer.)
     const int band = raster_div(pos / kGroupM, gn_magic);     // pos / (kGroupM * GN)
     const int first_m = band * kGroupM;
     const int in_band = pos - band * kGroupM * GN;
+    const int rows = GM - first_m >= kGroupM ? kGroupM : GM - first_m;
+    const int block = in_band / (rows * kUnitN);              // (only the band's last block can be narrower)
+    const int in_block = in_band - block * rows * kUnitN;
+    const int cols = GN - block * kUnitN >= kUnitN ? kUnitN : GN - block * kUnitN;
+    const int r = cols == kUnitN ? in_block / kUnitN : in_block / cols;
     TileCoord c;
-    if (GM - first_m >= kGroupM) {                            // a full band: shifts only
-        const int block = in_band / (kGroupM * kUnitN);
-        const int in_block = in_band % (kGroupM * kUnitN);
-        c.m = first_m + in_block % kGroupM;
-        c.n = block * kUnitN + in_block / kGroupM;
-    } else {
-        const int rows = GM - first_m;
-        const int block = in_band / (rows * kUnitN);
-        const int in_block = in_band - block * rows * kUnitN;
-        c.m = first_m + in_block % rows;
-        c.n = block * kUnitN + in_block / rows;
-    }
+    c.m = first_m + r;
+    c.n = block * kUnitN + (in_block - r * cols);
     return c;
 }
 
