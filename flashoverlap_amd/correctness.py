@@ -7,7 +7,7 @@
 Builds the plain row-parallel linear + RMSNorm and the overlapped linear +
 ReorderRMSNorm from the shape's tuning file (configs/m{M}n{N}k{K}_{gpu}.json, or
 a default record if there is none), runs both on the same input and prints the
-reference's verdict lines: all-ones operands and allclose(1e-2, 1e-2) for
+reference's result lines: all-ones operands and allclose(1e-2, 1e-2) for
 all_reduce, N(0, 0.5) operands, the element of largest difference and
 allclose(5e-2, 5e-2) for reduce_scatter.  With one GPU the collective of the
 plain layer is the identity and --world_size only selects the ReduceScatter

@@ -124,7 +124,7 @@ def test_monitor_sampling_and_vote_agree_with_the_raster(ready):
 
 @pytest.mark.parametrize("comm_op,ws,rank,dt", [("all_reduce", 1, 0, torch.float16), ("reduce_scatter", 8, 3, torch.bfloat16)])
 def test_correctness_examples(ready, tmp_path, comm_op, ws, rank, dt):
-    """The two example scripts of the reference as one command: its verdict lines, and True."""
+    """The two example scripts of the reference as one command: its result lines, and True."""
     from flashoverlap_amd import correctness
     M, N, K = 2048, 1024, 512
     cfg = _config(M, N, 1, 32, tmp_path)
